@@ -31,8 +31,12 @@ class DeviceCache:
             if g.paged:
                 shape = (n, g.pool.num_pages, g.need.num_kv_heads, manager.page_size, g.need.head_dim)
                 k = torch.full(shape, fill, dtype=dtype, device=device)
-                v = torch.full(shape, fill, dtype=dtype, device=device)
-                self.pools[g.index] = (k, v)
+                if g.need.values:
+                    v = torch.full(shape, fill, dtype=dtype, device=device)
+                    self.pools[g.index] = (k, v)
+                else:                       # one vector a token is key and value: the views' v is their k
+                    v = k
+                    self.pools[g.index] = (k,)
                 for i, cid in enumerate(g.cache_ids):
                     self.views[cid] = CacheView(cid, g.index, k=k[i], v=v[i])
             else:

@@ -61,7 +61,9 @@ class CacheManager:
         self.groups: List[CacheGroup] = []
         self.group_of_cache: Dict[int, int] = {}
         by_key: Dict[object, CacheGroup] = {}
-        for cid in sorted(needs):
+        # ids are integers (a mixer's cache) or tuples (the state of another part of a run):
+        # integers first, each kind in its own order
+        for cid in sorted(needs, key=lambda c: (0, c, ()) if isinstance(c, int) else (1, 0, tuple(c))):
             need = needs[cid]
             if need.kind not in ("paged_kv", "state"):
                 raise ValueError(f"cache {cid}: unknown need kind {need.kind!r}")

@@ -34,3 +34,42 @@ def preset(name: str, **overrides) -> OptHyperParam:
                         word_embed_proj_dim=hidden)
     fields.update(overrides)
     return OptHyperParam(**fields).validate()
+
+
+# ---- named sizes of the Zitupel family, for runs with random weights: the layer sizes of the
+# OPT model of the same name (width, heads, feed-forward width), so that the two can be set side
+# by side.  Of every four layers three are gated linear attention and one is latent attention;
+# every second latent layer borrows the latent of the one before it; the first layer's
+# feed-forward is dense, the others route every token to 2 of 16 experts of a quarter of the
+# dense width each.
+def zitupel_preset(name: str, **overrides):
+    from .zitupel_param import ZitupelHyperParam
+    key = name.lower().replace("-", "_")
+    size = key.split("_", 1)[1] if "_" in key else ""
+    if "opt_" + size not in _SIZES:
+        raise KeyError(f"invalid model name {name!r}; valid names: " +
+                       " ".join("zitupel_" + k.split("_", 1)[1] for k in _SIZES))
+    n_layers, hidden, heads, ffn = _SIZES["opt_" + size]
+    n_layers = int(overrides.pop("num_layers", n_layers))
+    dense_only = bool(overrides.pop("dense_only", False))
+    hd = hidden // heads
+    layers, last_owner = [], None
+    for i in range(n_layers):
+        if i % 4 == 3:
+            mixer = {"heads": heads, "dim": hd, "vdim": hd, "kv_rank": 128, "scale": float(hd) ** -0.5}
+            if last_owner is not None:
+                mixer["kv_from"], last_owner = last_owner, None
+            else:
+                last_owner = i
+            kind = "latent_attention"
+        else:
+            mixer, kind = {"heads": heads, "dim": hd, "vdim": hd, "tau": 16.0, "decay_rank": 16}, "gla"
+        if i == 0 or dense_only:
+            mlp = {"kind": "dense", "ff": ffn}
+        else:
+            mlp = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": ffn // 4, "limit": 7.0}}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    fields: Dict = dict(vocab=50272, width=hidden, layers=layers, residual_mult=0.5, norm_eps=1e-5, canon_taps=4,
+                        max_positions=2048)
+    fields.update(overrides)
+    return ZitupelHyperParam(**fields).validate()

@@ -56,8 +56,8 @@ def registered_architectures():
 
 
 def _ensure_builtin() -> None:
-    # the built-in architecture registers itself on import
-    from ..models import opt  # noqa: F401
+    # the built-in architectures register themselves on import
+    from ..models import opt, zitupel  # noqa: F401
 
 
 def resolve_architecture(name: str) -> Architecture:
@@ -80,6 +80,8 @@ def hyper_param_from_dir(model_dir: str):
     """(architecture, typed hyper-parameters) of the model in ``model_dir``."""
     cfg = read_config(model_dir)
     archs = cfg.get("architectures")
+    if not archs and isinstance(cfg.get("architecture"), str):
+        archs = [cfg["architecture"]]            # some families name their one class in the singular
     if archs:
         arch = resolve_architecture(archs[0])
     else:
@@ -89,7 +91,22 @@ def hyper_param_from_dir(model_dir: str):
         matches = [a for a in _ARCHITECTURES.values() if a.short_name and a.short_name == family]
         if not matches:
             raise ConfigError("config.json names no architecture: neither 'architectures' nor a known "
-                              f"'model_type' (registered: {sorted(_ARCHITECTURES)})")
+                              f"'architecture' nor a known 'model_type' (registered: {sorted(_ARCHITECTURES)})")
         arch = matches[0]
         cfg = dict(cfg, architectures=[arch.name])
-    return arch, arch.hyper_param_cls.from_dict(cfg)
+    hp = arch.hyper_param_cls.from_dict(cfg)
+    if hasattr(hp, "with_tensor_shapes"):
+        # sizes that config.json leaves to the tensors' shapes: read from the weight file's header
+        hp = hp.with_tensor_shapes(_shape_lookup(model_dir))
+    return arch, hp
+
+
+def _shape_lookup(model_dir: str):
+    files = []
+
+    def shape_of(name: str):
+        if not files:
+            from ..weights.safetensors_io import ModelFiles
+            files.append(ModelFiles(model_dir))
+        return tuple(files[0].shape(name)) if name in files[0] else None
+    return shape_of

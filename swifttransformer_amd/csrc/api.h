@@ -38,7 +38,7 @@ int st_activation_multiply(void* out, int64_t out_stride, const void* a, int64_t
 
 struct StGemmExtras;
 // activation: the function between bias and residual, by number (csrc/activation.h): 0 none,
-// 1 ReLU, 2 SiLU, 3 GELU in its tanh form; others are refused.
+// 1 ReLU, 2 SiLU, 3 GELU in its tanh form, 4 GELU in its exact (erf) form; others are refused.
 int st_gemm(void* out, const void* x, const void* w, const float* bias, const float* residual,
             int M, int N, int K, int activation, int dtype, int out_f32, int algo,
             const StGemmExtras* extras, hipStream_t stream);
@@ -97,6 +97,66 @@ int st_sample(int* out, const float* logits, int num_rows, int vocab, const floa
               const uint32_t* seeds, const uint32_t* draws, hipStream_t stream);
 
 float st_hash_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t draw, uint32_t v);
+
+// ---- short causal convolution over time, one filter a channel (csrc/token_conv.hip)
+// out[t, c] = x[t, c] + sum_j w[c, j] * x(row of position p_t - taps + 1 + j, c): rows before the
+// item's first row of this step come from state[slot, taps - 1, channels] (the inputs at the last
+// taps - 1 positions before it; zeros before the sequence's start).  st_token_conv_state then moves
+// the state on by the step's rows.  Rows whose item is -1 are written as zeros.
+int st_token_conv(void* out, const float* x, const float* w, const float* state, const int* token_item,
+                  const int* item_tok_off, const int* item_slot, int num_tokens, int channels, int taps,
+                  int add_input, int out_dtype, hipStream_t stream);
+int st_token_conv_state(float* state, const float* x, const int* item_len, const int* item_tok_off,
+                        const int* item_slot, int num_items, int channels, int taps, hipStream_t stream);
+
+// ---- gated linear attention (csrc/recurrent.hip)
+// a = sigmoid(z)^(inv_tau), in place over n floats.
+int st_decay_gate(float* z, int64_t n, float inv_tau, hipStream_t stream);
+// Per item and head, from the state S [key_dim, value_dim] of the item's slot and over its rows in
+// order: S = diag(a_t) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.  q, k, v:
+// rows of `dtype` with their strides in elements (head h at h * key_dim / h * value_dim); a: float
+// [T, heads * key_dim]; o: float [T, heads * value_dim]; state: float [slots, heads, key_dim, value_dim].
+int st_gla_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
+                const void* v, int64_t v_stride, const float* a, float* state,
+                const int* item_len, const int* item_tok_off, const int* item_slot, int num_items,
+                int heads, int key_dim, int value_dim, float scale, int dtype, hipStream_t stream);
+// out[t, h, j] = o[t, h, j] * rsqrt(mean_j o[t, h, :]^2 + eps) * gain[j] * silu(g[t, h, j]); g: rows
+// of `dtype` with stride g_stride; out: rows of `dtype`, dense.
+int st_gated_head_norm(void* out, const float* o, const void* g, int64_t g_stride, const float* gain,
+                       int num_tokens, int heads, int value_dim, float eps, int dtype, hipStream_t stream);
+
+// ---- latent cache (csrc/latent.hip)
+// Row t of x (float, stride x_stride, `rank` values) is normalised, c = x * rsqrt(mean x^2 + eps) *
+// gain, and stored as the token's entry of a one-head page pool whose entries are `entry` >= rank
+// wide (the rest is cleared): [pages, 1, page_size, entry] of `dtype`.
+int st_latent_write(void* cache, int64_t page_stride, const float* x, int64_t x_stride, const float* gain,
+                    const int* token_item, const int* positions, const int* block_table, int max_pages,
+                    int page_size, int num_tokens, int rank, int entry, float eps, int dtype, hipStream_t stream);
+
+// ---- routed experts (csrc/moe.hip)
+// ids[t, j], weights[t, j] (j < top): the experts with the largest logits of row t, largest first,
+// the lower index on ties, and sigmoid of their logits.  Rows whose item is -1 get ids of -1.
+int st_moe_route(int* ids, float* weights, const float* logits, const int* token_item, int num_tokens,
+                 int experts, int top, hipStream_t stream);
+// Sorts the num_pairs = tokens * top (token, choice) pairs by expert into tiles of 16 entries that
+// hold one expert's pairs each: sorted[capacity] (pair index, or -1), place_of_pair[num_pairs]
+// (or -1), tile_expert[capacity / 16] (or -1).  capacity >= round_up(num_pairs, 16) + 16 * experts.
+int st_moe_align(int* sorted, int* place_of_pair, int* tile_expert, const int* ids, int num_pairs,
+                 int experts, int capacity, hipStream_t stream);
+// y[place, f] = g * sigmoid(1.702 g) * (u + 1) with g = min(s * (x_t . Wg[e, f]), limit) and
+// u = clamp(s * (x_t . Wu[e, f]), -limit, limit), for the pair (t, j) at `place`, e its expert and s
+// its weight.  x: [T, width]; w_gate, w_up: [experts, inner, width]; y: [capacity, inner].
+int st_moe_up(void* y, const void* x, const void* w_gate, const void* w_up, const int* sorted,
+              const int* tile_expert, const float* weights, int capacity, int top, int width, int inner,
+              float limit, int dtype, hipStream_t stream);
+// pair_out[place, n] = y[place] . Wd[e, n] (top > 1), or, with top == 1, directly
+// out[t, n] = residual[t, n] + out_scale * y[place] . Wd[e, n].  w_down: [experts, width, inner].
+int st_moe_down(float* out, const float* residual, float* pair_out, const void* y, const void* w_down,
+                const int* sorted, const int* tile_expert, int capacity, int top, int width, int inner,
+                float out_scale, int dtype, hipStream_t stream);
+// out[t, n] = residual[t, n] + out_scale * sum_j pair_out[place_of_pair[t * top + j], n]
+int st_moe_combine(float* out, const float* residual, const float* pair_out, const int* place_of_pair,
+                   int num_tokens, int top, int width, float out_scale, hipStream_t stream);
 
 // Measurement kernels (csrc/probe.hip): a plain streaming read, and a kernel without work.
 int st_probe_read(const void* src, int64_t bytes, void* sink, int workgroups, int pattern, hipStream_t stream);

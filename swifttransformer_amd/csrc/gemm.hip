@@ -71,6 +71,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
             float v = acc[i][j];
             if (bias) v += bias[n];
             v = apply_activation(act, v);
+            if (ex.out_scale != 0.f) v *= ex.out_scale;
             if (residual) v += residual[(int64_t)m * N + n];
             Elem<TO>::store(out + (int64_t)m * N + n, v);
             if (ex.k_cache && n >= ex.q_size) {
@@ -103,7 +104,7 @@ int gemm_wide_groups();
 int gemm_wide(float* out, const bf16_t* x, const bf16_t* w, const float* bias, int M, int N, int K,
               const StGemmExtras& ex, hipStream_t stream);
 int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                 int M, int N, int K, int act, int out_f32, int dtype, hipStream_t stream, bool* handled);
+                 int M, int N, int K, int act, int out_f32, int dtype, float alpha, hipStream_t stream, bool* handled);
 
 // Float products always go to the library when it has a kernel (the float kernel here is the
 // plain tiled one).  For bfloat16:
@@ -144,7 +145,7 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
                        int out_f32, int algo, const StGemmExtras* extras, hipStream_t stream) {
     ST_CHECK(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     ST_CHECK(activation_known(activation), "gemm: activation %d has no kernel (0 none, 1 ReLU, 2 SiLU, "
-             "3 GELU in its tanh form)", activation);
+             "3 GELU in its tanh form, 4 GELU in its exact form)", activation);
     const int act = activation;
     StGemmExtras ex = {};
     if (extras) ex = *extras;
@@ -157,9 +158,11 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
         ST_CHECK(!out_f32 || dtype == kF32, "gemm: K/V scatter stores the storage type");
         ST_CHECK(!act && !residual, "gemm: K/V scatter goes with a plain product");
     }
+    if (ex.out_scale == 1.f) ex.out_scale = 0.f;
+    const bool scaled = ex.out_scale != 0.f;
     if (M == 0) return 0;
     // the persistent kernel for a few rows and a very wide matrix: float results of a plain product
-    const bool wide_can = dtype == kBF16 && out_f32 && !residual && act == 0 && !ex.k_cache && !ex.mg_o &&
+    const bool wide_can = dtype == kBF16 && out_f32 && !residual && act == 0 && !ex.k_cache && !ex.mg_o && !scaled &&
                           (algo == 0 || algo == 3) && K % 8 == 0 && gemm_wide_offered(M, N, K) &&
                           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
                             reinterpret_cast<uintptr_t>(ex.ln_x) | reinterpret_cast<uintptr_t>(ex.ln_gamma) |
@@ -190,14 +193,15 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
     // elementwise kernel after the library's product (a product with a residual sum cannot be
     // split like that and stays with the kernels here).
     const bool in_epilogue = activation_in_library(act);
-    const bool library_can = in_epilogue || !residual;
+    const bool library_can = (in_epilogue || !residual) && (!scaled || (act == 0 && !bias));
     ST_CHECK(algo != 2 || library_can, "gemm: the library path has no activation %d before a residual sum", act);
     const bool to_library = algo == 2 || (algo == 0 && !ex.ln_x && !ex.mg_o && library_can &&
         (dtype == kF32 || M >= g_library_min_rows ||
          ((int64_t)N * K >= g_library_min_weights && K >= g_library_min_depth)));
     if (to_library && (dtype == kF32 || dtype == kBF16)) {
         bool handled = false;
-        int rc = gemm_library(out, x, w, bias, residual, M, N, K, in_epilogue ? act : 0, out_f32, dtype, stream, &handled);
+        int rc = gemm_library(out, x, w, bias, residual, M, N, K, in_epilogue ? act : 0, out_f32, dtype,
+                              scaled ? ex.out_scale : 1.f, stream, &handled);
         if (rc != 0) return rc;
         ST_CHECK(handled || algo != 2, "gemm: the library has no kernel for M=%d N=%d K=%d", M, N, K);
         if (handled) {

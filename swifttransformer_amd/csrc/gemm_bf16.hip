@@ -50,6 +50,10 @@ __device__ inline void store4(void* out, const float* bias, const float* residua
             if (n0 + i < N) r[i] += bias[n0 + i];
     }
     apply_activation4(act, r);
+    if (ex.out_scale != 0.f) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] *= ex.out_scale;
+    }
     if (residual) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)

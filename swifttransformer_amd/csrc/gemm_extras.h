@@ -11,6 +11,8 @@
 //    The persistent wide-matrix kernel (gemm_wide.hip) also takes the rows through an index.
 //  * Best-of-row epilogue: the index of every row's largest output (greedy token choice over a
 //    vocabulary without another pass over the logits).  Only the persistent wide-matrix kernel.
+//  * Scaled result: out = residual + out_scale * act(x W^T + bias), for blocks whose branches
+//    enter the residual stream with a constant factor.
 //  * K/V scatter epilogue: output features [q_size, q_size + 2*kv_size) of a fused QKV
 //    product are the new tokens' keys and values; besides the normal store they go
 //    straight into their cache pages (the reference does this with a separate kernel,
@@ -54,6 +56,11 @@ extern "C" struct StGemmExtras {
     int* best_ids;
     float* best_val;
     int* best_idx;
+    // scaled result: what the product, bias and activation gave is multiplied by out_scale before
+    // the residual is added (0 means 1).  The kernels of gemm.hip and gemm_bf16.hip and the library
+    // (as its alpha, for products without bias and activation) offer it.
+    float out_scale;
+    int _pad3;
 };
 
 namespace st {

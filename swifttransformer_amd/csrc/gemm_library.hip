@@ -201,7 +201,7 @@ Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool res
 // Combinations the library's epilogue does not express in this engine's order (ReLU before
 // the residual sum, a residual into a bfloat16 result) are left to the caller's kernels.
 int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                 int M, int N, int K, int relu, int out_f32, int dtype, hipStream_t stream, bool* handled) {
+                 int M, int N, int K, int relu, int out_f32, int dtype, float alpha, hipStream_t stream, bool* handled) {
     *handled = false;
     if (relu != 0 && relu != 1) return 0;            // `relu` is the activation's number: none or ReLU here
     if ((relu && residual) || (residual && !out_f32 && dtype != kF32)) return 0;
@@ -245,7 +245,7 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
         if (!ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bp, sizeof(bp))))
             return 0;
     }
-    const float alpha = 1.f, beta = residual ? 1.f : 0.f;
+    const float beta = residual ? 1.f : 0.f;       // (alpha: the caller's factor on the product)
     const void* c = residual ? (const void*)residual : (const void*)out;
     const hipblasStatus_t s = hipblasLtMatmul(lib.handle, p.desc, &alpha, w, p.a, x, p.b, &beta, c, p.c,
                                               out, p.d, &p.algo, lib.workspace, p.workspace, stream);

@@ -1,0 +1,320 @@
+// Routed experts: every token sends its vector, scaled by a routing weight, through `top` of
+// `experts` small gated feed-forward layers.
+//
+// Everything stays on the device and has a fixed launch shape, so a step can be recorded:
+//   route    per token the `top` largest router logits and the sigmoid of each;
+//   align    the (token, choice) pairs sorted by expert into tiles of 16 places, a tile holding
+//            pairs of one expert only (places left over are marked -1);
+//   up       per tile and 64 inner features: both input products on the matrix cores, rows
+//            gathered through the sorted list, then clamp, gate and product of the two halves;
+//   down     per tile and 64 output features: the output product; with one expert a token the
+//            result goes straight into the residual stream, otherwise to a row per pair that
+//   combine  sums in the order of the token's choices.
+// A wave computes a 16 x 16 block of results with operands read straight from memory in the
+// matrix instruction's own layout (16 bytes a lane and step): with 16 rows a tile the products
+// are bound by the stream of expert weights, which every tile reads once.
+#include "api.h"
+#include "common.h"
+
+namespace st {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kTile = 16;
+constexpr int kMaxTop = 16;
+
+__global__ __launch_bounds__(256) void moe_route_kernel(
+    int* __restrict__ ids, float* __restrict__ weights, const float* __restrict__ logits,
+    const int* __restrict__ token_item, int num_tokens, int experts, int top) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= num_tokens) return;
+    if (token_item && token_item[t] < 0) {
+        for (int j = 0; j < top; ++j) { ids[(int64_t)t * top + j] = -1; weights[(int64_t)t * top + j] = 0.f; }
+        return;
+    }
+    const float* z = logits + (int64_t)t * experts;
+    int chosen[kMaxTop];
+    for (int j = 0; j < top; ++j) {
+        int best = -1;
+        float bv = 0.f;
+        for (int e = 0; e < experts; ++e) {
+            bool taken = false;
+            for (int u = 0; u < j; ++u) taken |= chosen[u] == e;
+            const float v = z[e];
+            if (!taken && (best < 0 || v > bv)) { best = e; bv = v; }
+        }
+        chosen[j] = best;
+        ids[(int64_t)t * top + j] = best;
+        weights[(int64_t)t * top + j] = 1.f / (1.f + expf(-bv));
+    }
+}
+
+// One workgroup: counts, padded offsets, then places.  Which place of its expert's tiles a pair
+// gets depends on the order of the atomics; a pair's result does not depend on its place.
+__global__ __launch_bounds__(1024) void moe_align_kernel(
+    int* __restrict__ sorted, int* __restrict__ place_of_pair, int* __restrict__ tile_expert,
+    const int* __restrict__ ids, int num_pairs, int experts, int capacity) {
+    extern __shared__ int lds[];
+    int* count = lds;                  // [experts]
+    int* offset = lds + experts;       // [experts + 1]
+    const int tid = threadIdx.x;
+    for (int e = tid; e < experts; e += 1024) count[e] = 0;
+    for (int i = tid; i < capacity; i += 1024) sorted[i] = -1;
+    for (int i = tid; i < capacity / kTile; i += 1024) tile_expert[i] = -1;
+    __syncthreads();
+    for (int p = tid; p < num_pairs; p += 1024) {
+        const int e = ids[p];
+        if (e >= 0) atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int e = 0; e < experts; ++e) {
+            offset[e] = run;
+            run += (count[e] + kTile - 1) / kTile * kTile;
+        }
+        offset[experts] = run;
+    }
+    __syncthreads();
+    for (int e = tid; e < experts; e += 1024) {
+        for (int i = offset[e] / kTile; i < offset[e + 1] / kTile; ++i) tile_expert[i] = e;
+        count[e] = offset[e];          // from here on: the next free place of the expert
+    }
+    __syncthreads();
+    for (int p = tid; p < num_pairs; p += 1024) {
+        const int e = ids[p];
+        int place = -1;
+        if (e >= 0) {
+            place = atomicAdd(&count[e], 1);
+            sorted[place] = p;
+        }
+        place_of_pair[p] = place;
+    }
+}
+
+// ---- operands in the matrix instructions' layout: lane (r16, g) holds, of row r16, the elements
+// k0 + 8g .. 8g+7 (bfloat16, one product of depth 32) or k0 + 4g .. 4g+3 (float, four products
+// of depth 4, the u-th taking element u of every lane).
+template <typename T> struct Frag;
+template <> struct Frag<bf16_t> {
+    static constexpr int kDepth = 32, kLane = 8;
+    bf16x8 v;
+    __device__ inline void load(const bf16_t* row, int k, int K, bool ok, bool vec) {
+        if (ok && vec && k + 8 <= K) {
+            v = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(row + k));
+        } else {
+            uint16_t e[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) e[i] = (ok && k + i < K) ? row[k + i].bits : (uint16_t)0;
+            v = __builtin_bit_cast(bf16x8, make_uint4(e[0] | ((uint32_t)e[1] << 16), e[2] | ((uint32_t)e[3] << 16),
+                                                      e[4] | ((uint32_t)e[5] << 16), e[6] | ((uint32_t)e[7] << 16)));
+        }
+    }
+    __device__ static inline floatx4 mma(const Frag& a, const Frag& b, floatx4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, c, 0, 0, 0);
+    }
+};
+template <> struct Frag<float> {
+    static constexpr int kDepth = 16, kLane = 4;
+    float v[4];
+    __device__ inline void load(const float* row, int k, int K, bool ok, bool vec) {
+        if (ok && vec && k + 4 <= K) {
+            const float4 x = *reinterpret_cast<const float4*>(row + k);
+            v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = (ok && k + i < K) ? row[k + i] : 0.f;
+        }
+    }
+    __device__ static inline floatx4 mma(const Frag& a, const Frag& b, floatx4 c) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[u], b.v[u], c, 0, 0, 0);
+        return c;
+    }
+};
+
+// grid (tiles, ceil(inner / 64)); wave w of the workgroup takes inner features f0 + 16 w .. +15.
+// Result layout of a wave: lane (r16, g) holds rows 4g .. 4g+3 of feature r16.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_up_kernel(
+    T* __restrict__ y, const T* __restrict__ x, const T* __restrict__ w_gate, const T* __restrict__ w_up,
+    const int* __restrict__ sorted, const int* __restrict__ tile_expert, const float* __restrict__ weights,
+    int top, int width, int inner, float limit, int vec) {
+    const int tile = blockIdx.x;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+    const int f = blockIdx.y * 64 + wave * 16 + r16;           // this lane's feature as an operand row
+    const bool f_ok = f < inner;
+    const int pair = sorted[tile * kTile + r16];               // this lane's token row as an operand row
+    const bool p_ok = pair >= 0;
+    const T* xr = x + (int64_t)(p_ok ? pair / top : 0) * width;
+    const T* gr = w_gate + ((int64_t)e * inner + (f_ok ? f : 0)) * width;
+    const T* ur = w_up + ((int64_t)e * inner + (f_ok ? f : 0)) * width;
+    floatx4 cg = {0.f, 0.f, 0.f, 0.f}, cu = {0.f, 0.f, 0.f, 0.f};
+    constexpr int D = Frag<T>::kDepth, L = Frag<T>::kLane;
+    for (int k0 = 0; k0 < width; k0 += D) {
+        Frag<T> a, bg, bu;
+        const int k = k0 + L * g;
+        a.load(xr, k, width, p_ok, vec);
+        bg.load(gr, k, width, f_ok, vec);
+        bu.load(ur, k, width, f_ok, vec);
+        cg = Frag<T>::mma(a, bg, cg);
+        cu = Frag<T>::mma(a, bu, cu);
+    }
+    if (!f_ok) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int place = tile * kTile + 4 * g + r;
+        const int p = sorted[place];
+        float out = 0.f;
+        if (p >= 0) {
+            const float s = weights[p];
+            const float gv = fminf(s * cg[r], limit);
+            const float uv = fminf(fmaxf(s * cu[r], -limit), limit);
+            out = gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f);
+        }
+        Elem<T>::store(y + (int64_t)place * inner + f, out);
+    }
+}
+
+// grid (tiles, ceil(width / 64)).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_kernel(
+    float* __restrict__ out, const float* __restrict__ residual, float* __restrict__ pair_out,
+    const T* __restrict__ y, const T* __restrict__ w_down, const int* __restrict__ sorted,
+    const int* __restrict__ tile_expert, int top, int width, int inner, float out_scale, int vec) {
+    const int tile = blockIdx.x;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+    const int n = blockIdx.y * 64 + wave * 16 + r16;
+    const bool n_ok = n < width;
+    const T* yr = y + (int64_t)(tile * kTile + r16) * inner;
+    const T* wr = w_down + ((int64_t)e * width + (n_ok ? n : 0)) * inner;
+    floatx4 c = {0.f, 0.f, 0.f, 0.f};
+    constexpr int D = Frag<T>::kDepth, L = Frag<T>::kLane;
+    for (int k0 = 0; k0 < inner; k0 += D) {
+        Frag<T> a, b;
+        const int k = k0 + L * g;
+        a.load(yr, k, inner, true, vec);
+        b.load(wr, k, inner, n_ok, vec);
+        c = Frag<T>::mma(a, b, c);
+    }
+    if (!n_ok) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int place = tile * kTile + 4 * g + r;
+        const int p = sorted[place];
+        if (p < 0) continue;
+        if (pair_out) {
+            pair_out[(int64_t)place * width + n] = c[r];
+        } else {                                               // one expert a token: p is the token
+            const int64_t at = (int64_t)p * width + n;
+            out[at] = fmaf(out_scale, c[r], residual[at]);
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(
+    float* __restrict__ out, const float* __restrict__ residual, const float* __restrict__ pair_out,
+    const int* __restrict__ place_of_pair, int top, int width, float out_scale) {
+    const int t = blockIdx.x;
+    for (int n = threadIdx.x; n < width; n += 256) {
+        float sum = 0.f;
+        bool any = false;
+        for (int j = 0; j < top; ++j) {
+            const int place = place_of_pair[(int64_t)t * top + j];
+            if (place >= 0) { sum += pair_out[(int64_t)place * width + n]; any = true; }
+        }
+        const int64_t at = (int64_t)t * width + n;
+        if (any) out[at] = fmaf(out_scale, sum, residual[at]);
+        else if (out != residual) out[at] = residual[at];
+    }
+}
+
+}  // namespace st
+
+using namespace st;
+
+extern "C" int st_moe_route(int* ids, float* weights, const float* logits, const int* token_item, int num_tokens,
+                            int experts, int top, hipStream_t stream) {
+    ST_CHECK(num_tokens >= 0 && experts > 0, "moe_route: bad sizes");
+    ST_CHECK(top >= 1 && top <= kMaxTop && top <= experts, "moe_route: 1 to %d experts a token (of %d), not %d",
+             kMaxTop, experts, top);
+    ST_CHECK(ids && weights && logits, "moe_route: null operand");
+    if (num_tokens == 0) return 0;
+    moe_route_kernel<<<(num_tokens + 255) / 256, 256, 0, stream>>>(ids, weights, logits, token_item, num_tokens,
+                                                                  experts, top);
+    ST_LAUNCH_CHECK("moe_route");
+    return 0;
+}
+
+extern "C" int st_moe_align(int* sorted, int* place_of_pair, int* tile_expert, const int* ids, int num_pairs,
+                            int experts, int capacity, hipStream_t stream) {
+    ST_CHECK(num_pairs >= 0 && experts > 0 && experts <= 4096, "moe_align: bad sizes (up to 4096 experts)");
+    ST_CHECK(capacity % kTile == 0 && capacity >= (num_pairs + kTile - 1) / kTile * kTile + kTile * experts,
+             "moe_align: %d places do not hold %d pairs of %d experts in tiles of %d", capacity, num_pairs, experts, kTile);
+    ST_CHECK(sorted && place_of_pair && tile_expert && ids, "moe_align: null operand");
+    moe_align_kernel<<<1, 1024, (2 * experts + 1) * sizeof(int), stream>>>(sorted, place_of_pair, tile_expert, ids,
+                                                                          num_pairs, experts, capacity);
+    ST_LAUNCH_CHECK("moe_align");
+    return 0;
+}
+
+static bool rows_vectorised(const void* a, const void* b, const void* c, int depth, int dtype) {
+    const int per = dtype == kF32 ? 4 : 8;
+    return depth % per == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+                                 reinterpret_cast<uintptr_t>(c)) & 15) == 0;
+}
+
+extern "C" int st_moe_up(void* y, const void* x, const void* w_gate, const void* w_up, const int* sorted,
+                         const int* tile_expert, const float* weights, int capacity, int top, int width, int inner,
+                         float limit, int dtype, hipStream_t stream) {
+    ST_CHECK(capacity > 0 && capacity % kTile == 0 && top >= 1 && width > 0 && inner > 0, "moe_up: bad sizes");
+    ST_CHECK(y && x && w_gate && w_up && sorted && tile_expert && weights, "moe_up: null operand");
+    const dim3 grid(capacity / kTile, (inner + 63) / 64);
+    ST_CHECK(grid.y <= 65535, "moe_up: too many inner features");
+    const int vec = rows_vectorised(x, w_gate, w_up, width, dtype);
+    if (dtype == kF32)
+        moe_up_kernel<float><<<grid, 256, 0, stream>>>((float*)y, (const float*)x, (const float*)w_gate,
+            (const float*)w_up, sorted, tile_expert, weights, top, width, inner, limit, vec);
+    else if (dtype == kBF16)
+        moe_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w_gate,
+            (const bf16_t*)w_up, sorted, tile_expert, weights, top, width, inner, limit, vec);
+    else ST_CHECK(false, "moe_up: unknown dtype %d", dtype);
+    ST_LAUNCH_CHECK("moe_up");
+    return 0;
+}
+
+extern "C" int st_moe_down(float* out, const float* residual, float* pair_out, const void* y, const void* w_down,
+                           const int* sorted, const int* tile_expert, int capacity, int top, int width, int inner,
+                           float out_scale, int dtype, hipStream_t stream) {
+    ST_CHECK(capacity > 0 && capacity % kTile == 0 && top >= 1 && width > 0 && inner > 0, "moe_down: bad sizes");
+    ST_CHECK(y && w_down && sorted && tile_expert, "moe_down: null operand");
+    ST_CHECK(pair_out ? true : (top == 1 && out && residual),
+             "moe_down: without a row per pair the result goes to the stream, for one expert a token only");
+    const dim3 grid(capacity / kTile, (width + 63) / 64);
+    ST_CHECK(grid.y <= 65535, "moe_down: too wide");
+    const int vec = rows_vectorised(y, w_down, w_down, inner, dtype);
+    if (dtype == kF32)
+        moe_down_kernel<float><<<grid, 256, 0, stream>>>(out, residual, pair_out, (const float*)y, (const float*)w_down,
+            sorted, tile_expert, top, width, inner, out_scale, vec);
+    else if (dtype == kBF16)
+        moe_down_kernel<bf16_t><<<grid, 256, 0, stream>>>(out, residual, pair_out, (const bf16_t*)y,
+            (const bf16_t*)w_down, sorted, tile_expert, top, width, inner, out_scale, vec);
+    else ST_CHECK(false, "moe_down: unknown dtype %d", dtype);
+    ST_LAUNCH_CHECK("moe_down");
+    return 0;
+}
+
+extern "C" int st_moe_combine(float* out, const float* residual, const float* pair_out, const int* place_of_pair,
+                              int num_tokens, int top, int width, float out_scale, hipStream_t stream) {
+    ST_CHECK(num_tokens >= 0 && top >= 1 && width > 0, "moe_combine: bad sizes");
+    ST_CHECK(out && residual && pair_out && place_of_pair, "moe_combine: null operand");
+    if (num_tokens == 0) return 0;
+    moe_combine_kernel<<<num_tokens, 256, 0, stream>>>(out, residual, pair_out, place_of_pair, top, width, out_scale);
+    ST_LAUNCH_CHECK("moe_combine");
+    return 0;
+}

@@ -417,7 +417,7 @@ def pages_that_fit(model: DecoderModel, page_size: int, fraction: float, device)
         raise ValueError(f"gpu_mem_fraction is a share of the free memory in (0, 1], not {fraction}")
     free, _total = torch.cuda.mem_get_info(torch.device(device))
     elem = 2 if model.dtype == torch.bfloat16 else 4
-    per_page = sum(2 * need.num_kv_heads * need.head_dim * page_size * elem
+    per_page = sum((2 if need.values else 1) * need.num_kv_heads * need.head_dim * page_size * elem
                    for need in model.cache_needs().values() if need.kind == "paged_kv")
     if per_page == 0:
         return 1

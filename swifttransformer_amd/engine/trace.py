@@ -27,7 +27,7 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.
 
 
 def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[str],
-           log: IO[str] = sys.stdout, page_size: int = 16, max_live: int = 8,
+           log: IO[str] = sys.stdout, page_size: int = 16, max_live: int = 4,
            device: str = "cuda:0") -> int:
     if dtype not in _DTYPES:
         raise ValueError(f"--dtype must be bfloat16 or float32, got {dtype!r}")

@@ -5,6 +5,7 @@ and with random weights in memory (``random_model``).  The reference's counterpa
 loader and ``initDummyWeight`` (src/csrc/model/gpt/gpt_weight.cc:235-326, :329-408)."""
 from .decoder import DecoderModel
 from . import opt  # noqa: F401  (registers OPTForCausalLM)
+from . import zitupel  # noqa: F401  (registers Zitupel)
 from .opt import build_opt_spec
 
 __all__ = ["DecoderModel", "build_opt_spec", "build_model", "load_model", "random_model"]

@@ -26,9 +26,17 @@ class Layer:
     mixer: object
     ffn_norm: object
     feed_forward: object
+    mixer_conv: object = None
 
     def parts(self):
-        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward) if p is not None)
+        return tuple(p for p in (self.mixer_norm, self.mixer_conv, self.mixer, self.ffn_norm, self.feed_forward)
+                     if p is not None)
+
+
+def conv_cache_id(run: int):
+    """The cache id of the state that the ``mixer_conv`` part of the schedule's ``run``-th entry
+    keeps: one per run of a layer, also where the run's mixer reads another run's cache."""
+    return (run, "mixer_conv")
 
 
 class DecoderModel:
@@ -51,7 +59,8 @@ class DecoderModel:
                 mixer_norm=opt("norm", ls.mixer_norm),
                 mixer=build_part("mixer", ls.mixer, H, dtype),
                 ffn_norm=opt("norm", ls.ffn_norm),
-                feed_forward=opt("feed_forward", ls.feed_forward))
+                feed_forward=opt("feed_forward", ls.feed_forward),
+                mixer_conv=opt("token_conv", getattr(ls, "mixer_conv", None)))
             needs = getattr(layer.arrangement, "needs", ())
             missing = [n for n in needs if getattr(layer, n) is None]
             if missing:
@@ -96,10 +105,14 @@ class DecoderModel:
 
     # -------------------------------------------------------------------- cache
     def cache_needs(self) -> Dict[int, CacheNeed]:
-        """cache id -> need, for every cache the schedule writes."""
-        needs: Dict[int, CacheNeed] = {}
-        for e in self.schedule:
-            need = self.layers[e.layer].mixer.cache_need()
+        """cache id -> need, for every cache the schedule writes: the mixers' under the schedule's
+        own ids (integers), the state of a run's ``mixer_conv`` part under ``conv_cache_id(run)``."""
+        needs: Dict[object, CacheNeed] = {}
+        for run, e in enumerate(self.schedule):
+            layer = self.layers[e.layer]
+            if layer.mixer_conv is not None:
+                needs[conv_cache_id(run)] = layer.mixer_conv.cache_need()
+            need = layer.mixer.cache_need()
             if need is None:
                 continue
             if e.cache in needs and needs[e.cache].group_key() != need.group_key():
@@ -137,10 +150,14 @@ class DecoderModel:
             raise RuntimeError("load the weights before running the model")
         ctx.position = self.position
         x32 = self.embedding.forward(ctx, self.position)
-        for e in self.schedule:
+        for run, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
             K.arena.next_bank()      # what this run of a layer makes may be read until the next one ends
-            x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write)
+            if layer.mixer_conv is not None:
+                x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write,
+                                                conv_cache=caches.get(conv_cache_id(run)))
+            else:
+                x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write)
         return x32
 
     def forward_head(self, x32: torch.Tensor, ctx, want_rows: Optional[torch.Tensor] = None,

@@ -65,6 +65,22 @@ def _lib():
         lib.st_probe_fill.argtypes = [_c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_p]
         lib.st_probe_mfma.argtypes = [_c_p, _c_int, _c_int, _c_int, _c_p]
         lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
+        lib.st_token_conv.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int,
+                                      _c_int, _c_p]
+        lib.st_token_conv_state.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_decay_gate.argtypes = [_c_p, _c_i64, _c_f, _c_p]
+        lib.st_gla_scan.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p,
+                                    _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_gated_head_norm.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_latent_write.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
+                                        _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_moe_route.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_moe_align.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_moe_up.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_f,
+                                  _c_int, _c_p]
+        lib.st_moe_down.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_f,
+                                    _c_int, _c_p]
+        lib.st_moe_combine.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_f, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
         _configured = True
@@ -225,7 +241,8 @@ class _GemmExtras(ctypes.Structure):
                 ("q_size", _c_int), ("kv_size", _c_int), ("head_dim", _c_int), ("_pad1", _c_int),
                 ("mg_o", _c_p), ("mg_lse", _c_p), ("mg_splits", _c_int), ("mg_heads", _c_int),
                 ("mg_head_dim", _c_int), ("_pad2", _c_int),
-                ("ln_rows", _c_p), ("best_ids", _c_p), ("best_val", _c_p), ("best_idx", _c_p)]
+                ("ln_rows", _c_p), ("best_ids", _c_p), ("best_val", _c_p), ("best_idx", _c_p),
+                ("out_scale", _c_f), ("_pad3", _c_int)]
 
 
 class KvScatter:
@@ -323,11 +340,11 @@ def wide_offered(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
 
 # functions of the products' epilogues and of ``activation_multiply``, by the C interface's number
 # (csrc/activation.h; the names config files use for them)
-ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3}
+ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3, "gelu": 4, "gelu_erf": 4}
 
 
 def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_f32=False, algo=0,
-            kv_scatter=None, best=None):
+            kv_scatter=None, best=None, out_scale=1.0):
     N, K = w.shape
     fused = []
     if isinstance(x, NormInput):
@@ -357,9 +374,10 @@ def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_
 def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
          residual: Optional[torch.Tensor] = None, activation: str = "none",
          out: Optional[torch.Tensor] = None, out_f32: bool = False, algo: int = 0,
-         kv_scatter: Optional[KvScatter] = None, best: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[M,N] = act(x[M,K] @ w[N,K]^T (+bias)) (+residual); float accumulation.  ``activation``
-    is one of ``ACTIVATIONS``.
+         kv_scatter: Optional[KvScatter] = None, best: Optional[torch.Tensor] = None,
+         out_scale: float = 1.0) -> torch.Tensor:
+    """out[M,N] = out_scale * act(x[M,K] @ w[N,K]^T (+bias)) (+residual); float accumulation.
+    ``activation`` is one of ``ACTIVATIONS``.
 
     ``x`` is a tensor of w's dtype, a ``NormInput`` (where ``can_fuse_norm``) or a
     ``SplitAttention`` (where ``can_fuse_merge``).  With
@@ -430,6 +448,10 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
         idx = empty((n_scratch,), torch.int32, device)
         keep += [val, idx]
         ex.best_ids, ex.best_val, ex.best_idx = _ptr(best), _ptr(val), _ptr(idx)
+    if float(out_scale) != 1.0:
+        if ex is None:
+            ex = _GemmExtras()
+        ex.out_scale = float(out_scale)
     _check(_lib().st_gemm(_ptr(out), x_ptr, _ptr(w), _ptr(bias), _ptr(residual), M, N, K, ACTIVATIONS[activation],
                           code, int(odt == torch.float32), int(algo),
                           ctypes.byref(ex) if ex is not None else None, _stream()))
@@ -698,6 +720,186 @@ def activation(x: torch.Tensor, kind: str, out: Optional[torch.Tensor] = None) -
 def multiply(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = a * b elementwise."""
     return activation_multiply(a, b, "none", out)
+
+
+# ------------------------------------------------- short convolution over time
+def _d_token_conv(x, weight, state, ctx_arrays, out_dtype, **kw):
+    n, c = x.shape
+    return {"rows": n, "width": c, "bytes": n * c * (4 + torch.empty((), dtype=out_dtype).element_size())}
+
+
+@_timed("token_conv", _d_token_conv)
+def token_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx_arrays, out_dtype: torch.dtype,
+               add_input: bool = True, update_state: bool = True) -> torch.Tensor:
+    """y[t] = (x[t] if add_input) + sum_j weight[:, j] * x(position of t - taps + 1 + j) per channel,
+    over the rows of a batch: what lies before an item's first row is read from ``state``
+    [slots, taps - 1, channels] (float), which is then moved on by the item's rows.
+
+    x: float [T, channels]; weight: float [channels, taps]; ``ctx_arrays``: the batch's
+    (token_item, item_len, item_tok_off, item_slot)."""
+    token_item, item_len, item_tok_off, item_slot = ctx_arrays
+    T, C = x.shape
+    taps = weight.shape[1]
+    _need(x, "x", torch.float32, (T, C))
+    _need(weight, "weight", torch.float32, (C, taps))
+    _need(state, "state", torch.float32, (state.shape[0], max(taps - 1, 0), C))
+    _need(token_item, "token_item", torch.int32, (T,))
+    B = item_slot.shape[0]
+    for name, v in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
+        _need(v, name, torch.int32, (B,))
+    out = empty((T, C), out_dtype, x.device)
+    _check(_lib().st_token_conv(_ptr(out), _ptr(x), _ptr(weight), _ptr(state), _ptr(token_item), _ptr(item_tok_off),
+                                _ptr(item_slot), T, C, taps, int(bool(add_input)), dtype_code(out_dtype), _stream()))
+    if update_state:
+        _check(_lib().st_token_conv_state(_ptr(state), _ptr(x), _ptr(item_len), _ptr(item_tok_off), _ptr(item_slot),
+                                          B, C, taps, _stream()))
+    return out
+
+
+# ------------------------------------------------------ gated linear attention
+def decay_gate(z: torch.Tensor, inv_tau: float) -> torch.Tensor:
+    """In place: z <- sigmoid(z) ** inv_tau (float), computed as exp(inv_tau * log sigmoid(z))."""
+    _need(z, "z", torch.float32)
+    _check(_lib().st_decay_gate(_ptr(z), z.numel(), float(inv_tau), _stream()))
+    return z
+
+
+def _d_gla_scan(q, k, v, decay, state, ctx_arrays, heads, scale):
+    T = q.shape[0]
+    kd, vd = q.shape[1] // heads, v.shape[1] // heads
+    return {"rows": T, "heads": heads, "key_dim": kd, "value_dim": vd, "items": ctx_arrays[2].shape[0],
+            "flops": 4 * T * heads * kd * vd,
+            "bytes": T * heads * ((2 * kd + vd) * q.element_size() + 4 * kd + 4 * vd)}
+
+
+@_timed("gla_scan", _d_gla_scan)
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
+             ctx_arrays, heads: int, scale: float) -> torch.Tensor:
+    """Per item and head, from the slot's state S and over the item's rows in order:
+    S <- diag(decay_t) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.
+
+    q, k: [T, heads * key_dim], v: [T, heads * value_dim] views (dense rows, any row stride);
+    decay: float [T, heads * key_dim]; state: float [slots, heads, key_dim, value_dim].  Returns
+    float [T, heads * value_dim]."""
+    _token_item, item_len, item_tok_off, item_slot = ctx_arrays
+    T = q.shape[0]
+    kd, vd = q.shape[1] // heads, v.shape[1] // heads
+    for name, t, w in (("q", q, heads * kd), ("k", k, heads * kd), ("v", v, heads * vd)):
+        _need(t, name, q.dtype, (T, w), contiguous=False)
+        if t.stride(1) != 1:
+            raise KernelError(f"{name}: rows must be dense")
+    _need(decay, "decay", torch.float32, (T, heads * kd))
+    _need(state, "state", torch.float32, (state.shape[0], heads, kd, vd))
+    B = item_slot.shape[0]
+    for name, t in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
+        _need(t, name, torch.int32, (B,))
+    out = empty((T, heads * vd), torch.float32, q.device)
+    _check(_lib().st_gla_scan(_ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
+                              _ptr(decay), _ptr(state), _ptr(item_len), _ptr(item_tok_off), _ptr(item_slot), B,
+                              heads, kd, vd, float(scale), dtype_code(q.dtype), _stream()))
+    return out
+
+
+def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, heads: int, eps: float,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """out[t, h, :] = o[t, h, :] * rsqrt(mean(o[t, h, :]^2) + eps) * gain * silu(gate[t, h, :]).
+    o: float [T, heads * value_dim]; gate: a view of ``out_dtype`` rows; gain: float [value_dim]."""
+    T = o.shape[0]
+    vd = o.shape[1] // heads
+    _need(o, "o", torch.float32, (T, heads * vd))
+    _need(gate, "gate", out_dtype, (T, heads * vd), contiguous=False)
+    if gate.stride(1) != 1:
+        raise KernelError("gate: rows must be dense")
+    _need(gain, "gain", torch.float32, (vd,))
+    out = empty((T, heads * vd), out_dtype, o.device)
+    _check(_lib().st_gated_head_norm(_ptr(out), _ptr(o), _ptr(gate), gate.stride(0), _ptr(gain), T, heads, vd,
+                                     float(eps), dtype_code(out_dtype), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ latent cache
+def latent_write(cache: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, token_item: torch.Tensor,
+                 positions: torch.Tensor, block_table: torch.Tensor) -> None:
+    """Each row of x (float [T, rank], dense rows of any stride) is normalised to unit root mean
+    square, multiplied by ``gain`` and stored as its token's entry of ``cache``
+    [pages, 1, page_size, entry] with entry >= rank (the rest of an entry is cleared)."""
+    num_pages, one, ps, entry = cache.shape
+    T, rank = x.shape
+    _need(cache, "cache", None, (num_pages, 1, ps, entry), contiguous=False)
+    if cache.stride()[1:] != (ps * entry, entry, 1) or entry < rank:
+        raise KernelError("latent_write: pages of one head must be contiguous and an entry as wide as the rank")
+    _need(x, "x", torch.float32, (T, rank), contiguous=False)
+    if x.stride(1) != 1:
+        raise KernelError("x: rows must be dense")
+    _need(gain, "gain", torch.float32, (rank,))
+    _need(token_item, "token_item", torch.int32, (T,))
+    _need(positions, "positions", torch.int32, (T,))
+    _need(block_table, "block_table", torch.int32)
+    _check(_lib().st_latent_write(_ptr(cache), cache.stride(0), _ptr(x), x.stride(0), _ptr(gain), _ptr(token_item),
+                                  _ptr(positions), _ptr(block_table), block_table.shape[1], ps, T, rank, entry,
+                                  float(eps), dtype_code(cache.dtype), _stream()))
+
+
+# ---------------------------------------------------------------- routed experts
+MOE_TILE = 16
+
+
+def moe_capacity(num_tokens: int, top: int, experts: int) -> int:
+    """Places of the sorted pair list: every expert's pairs start a tile of their own."""
+    return -(-num_tokens * top // MOE_TILE) * MOE_TILE + MOE_TILE * experts
+
+
+def _d_moe(x, logits, w_gate, w_up, w_down, residual, *, top, limit, out_scale=1.0, token_item=None):
+    T, W = x.shape
+    E, F, _ = w_gate.shape
+    used = min(E, T * top)
+    return {"rows": T, "width": W, "inner": F, "experts": E, "top": top,
+            "flops": 6 * T * top * W * F, "bytes": used * 3 * F * W * x.element_size() + T * W * (x.element_size() + 8)}
+
+
+@_timed("routed_experts", _d_moe)
+def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
+                   w_down: torch.Tensor, residual: torch.Tensor, *, top: int, limit: float, out_scale: float = 1.0,
+                   token_item: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """residual <- residual + out_scale * sum over a row's ``top`` best experts e (by ``logits``) of
+    Wd[e] y with y = g * sigmoid(1.702 g) * (u + 1), g = min(s * Wg[e] x, limit),
+    u = clamp(s * Wu[e] x, -limit, limit), s = sigmoid(logit of e).  In place on ``residual``
+    (float [T, width]), which is returned.
+
+    x: [T, width]; logits: float [T, experts]; w_gate, w_up: [experts, inner, width]; w_down:
+    [experts, width, inner].  Rows whose ``token_item`` is negative are left as they are."""
+    T, W = x.shape
+    E, F, _ = w_gate.shape
+    _need(x, "x", w_gate.dtype, (T, W))
+    _need(logits, "logits", torch.float32, (T, E))
+    _need(w_gate, "w_gate", None, (E, F, W))
+    _need(w_up, "w_up", w_gate.dtype, (E, F, W))
+    _need(w_down, "w_down", w_gate.dtype, (E, W, F))
+    _need(residual, "residual", torch.float32, (T, W))
+    if token_item is not None:
+        _need(token_item, "token_item", torch.int32, (T,))
+    lib, dev, code, st = _lib(), x.device, dtype_code(x.dtype), _stream()
+    cap = moe_capacity(T, top, E)
+    ids = empty((T * top,), torch.int32, dev)
+    wts = empty((T * top,), torch.float32, dev)
+    sorted_pairs = empty((cap,), torch.int32, dev)
+    place = empty((T * top,), torch.int32, dev)
+    tile_expert = empty((cap // MOE_TILE,), torch.int32, dev)
+    y = empty((cap, F), x.dtype, dev)
+    _check(lib.st_moe_route(_ptr(ids), _ptr(wts), _ptr(logits), _ptr(token_item), T, E, int(top), st))
+    _check(lib.st_moe_align(_ptr(sorted_pairs), _ptr(place), _ptr(tile_expert), _ptr(ids), T * top, E, cap, st))
+    _check(lib.st_moe_up(_ptr(y), _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(sorted_pairs), _ptr(tile_expert),
+                         _ptr(wts), cap, int(top), W, F, float(limit), code, st))
+    if top == 1:
+        _check(lib.st_moe_down(_ptr(residual), _ptr(residual), None, _ptr(y), _ptr(w_down), _ptr(sorted_pairs),
+                               _ptr(tile_expert), cap, 1, W, F, float(out_scale), code, st))
+    else:
+        pair_out = empty((cap, W), torch.float32, dev)
+        _check(lib.st_moe_down(None, None, _ptr(pair_out), _ptr(y), _ptr(w_down), _ptr(sorted_pairs),
+                               _ptr(tile_expert), cap, int(top), W, F, float(out_scale), code, st))
+        _check(lib.st_moe_combine(_ptr(residual), _ptr(residual), _ptr(pair_out), _ptr(place), T, int(top), W,
+                                  float(out_scale), st))
+    return residual
 
 
 def probe_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, pattern: int = 0) -> None:

@@ -2,6 +2,8 @@
 
 pre-norm (reference src/csrc/model/gpt/gpt.cc:325-335, :347-391, :423-436, :467-501):
     a = N1(x); r = x + Mix(a); d = N2(r); x' = r + FFN(d)
+    (optionally a = C(N1(x)) with C a short filter over time, and optionally without the second
+    half; a factor on the branches is the mixer's and the feed-forward's own parameter)
 post-norm (the reference refuses it, gpt.cc:238-240):
     r = N1(x + Mix(x)); x' = N2(r + FFN(r))
 The residual stream is float; parts that multiply matrices take the storage type."""
@@ -20,15 +22,29 @@ def _fuses(part, norm, rows: int) -> bool:
 
 
 class PreNorm(Part):
-    needs = ("mixer_norm", "ffn_norm", "feed_forward")    # layer slots that must be filled
+    """params: feed_forward (bool, default True; False: the block ends after the mixer).  A layer
+    with a ``mixer_conv`` part has its mixer read conv(N1(x)) instead of N1(x)."""
 
-    def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True) -> torch.Tensor:
+    def __init__(self, spec, hidden_size, dtype):
+        super().__init__(spec, hidden_size, dtype)
+        self.has_ffn = bool(spec.params.get("feed_forward", True))
+        # layer slots that must be filled
+        self.needs = ("mixer_norm", "ffn_norm", "feed_forward") if self.has_ffn else ("mixer_norm",)
+
+    def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True, conv_cache=None) -> torch.Tensor:
         rows = x32.shape[0]
-        if _fuses(layer.mixer, layer.mixer_norm, rows):
+        if layer.mixer_conv is not None:
+            # the filter reads the float norm and makes the mixer's input in the storage type
+            _, n32 = layer.mixer_norm.forward(x32, out_t=False, out_f32=True)
+            a = layer.mixer_conv.forward(n32, ctx, conv_cache)
+            r32 = layer.mixer.forward(a, x32, ctx, cache, write)
+        elif _fuses(layer.mixer, layer.mixer_norm, rows):
             r32 = layer.mixer.forward(None, x32, ctx, cache, write, norm=layer.mixer_norm)
         else:
             a, _ = layer.mixer_norm.forward(x32, out_t=True)
             r32 = layer.mixer.forward(a, x32, ctx, cache, write)
+        if not self.has_ffn:
+            return r32
         if _fuses(layer.feed_forward, layer.ffn_norm, rows):
             return layer.feed_forward.forward(None, r32, ctx, norm=layer.ffn_norm)
         d, _ = layer.ffn_norm.forward(r32, out_t=True)

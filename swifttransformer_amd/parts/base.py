@@ -24,7 +24,10 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
                 scores when ``biases_scores`` is true
   embedding     ``forward(ctx, position) -> x32``
   head          ``forward(y_t) -> logits float32 [R, vocab]``
-  arrangement   ``forward(x32, layer, ctx, cache, write) -> x32``
+  arrangement   ``forward(x32, layer, ctx, cache, write) -> x32`` (with ``conv_cache=`` for a layer
+                that has a ``mixer_conv`` part)
+  token_conv    ``cache_need() -> CacheNeed``; ``forward(y32, ctx, cache) -> y_t``: a short causal
+                filter over time on what a mixer reads, with its last inputs as per-request state
 
 Any part may also offer ``step_planner() -> (key, planner)``: ``planner(items, info)`` sees the
 step's items on the host (slot, start, tokens of each) and a ``BatchInfo`` and returns a
@@ -45,7 +48,7 @@ import torch
 from ..weights.loader import TensorSpec
 from .spec import PartSpec
 
-CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "arrangement")
+CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "arrangement", "token_conv")
 _REGISTRY: Dict[str, Dict[str, Callable]] = {c: {} for c in CATEGORIES}
 
 
@@ -71,7 +74,8 @@ class CacheNeed:
 
     kind "paged_kv": keys and values in pages, ``num_kv_heads * head_dim`` elements
     per token each; ``window`` > 0 means only the last ``window`` tokens are ever
-    read, so pages behind it are given back.
+    read, so pages behind it are given back.  ``values`` False: one vector per token serves as
+    key and as value (a latent cache); no second pool is allocated and the view's ``v`` is its ``k``.
     kind "state": a fixed-size tensor per request (``state_shape``, ``state_dtype``),
     living in the request's state slot."""
     kind: str
@@ -80,10 +84,11 @@ class CacheNeed:
     window: int = 0
     state_shape: Tuple[int, ...] = ()
     state_dtype: Optional[torch.dtype] = None
+    values: bool = True
 
     def group_key(self):
         return (self.kind, self.num_kv_heads, self.head_dim, self.window, self.state_shape,
-                self.state_dtype)
+                self.state_dtype, self.values)
 
 
 @dataclass

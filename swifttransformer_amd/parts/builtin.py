@@ -6,6 +6,10 @@ from .embedding import TokenEmbedding, LMHead
 from .feed_forward import DenseFeedForward
 from .attention import PagedAttention
 from .arrangement import PreNorm, PostNorm
+from .conv import CausalTokenConv
+from .linear_attention import GatedLinearAttention
+from .latent_attention import LatentAttention
+from .routed import RoutedExperts
 
 register_part("norm", "layer_norm", LayerNorm)
 register_part("position", "learned", LearnedPositions)
@@ -16,3 +20,7 @@ register_part("feed_forward", "dense", DenseFeedForward)
 register_part("mixer", "paged_attention", PagedAttention)
 register_part("arrangement", "pre_norm", PreNorm)
 register_part("arrangement", "post_norm", PostNorm)
+register_part("token_conv", "causal", CausalTokenConv)
+register_part("mixer", "gated_linear_attention", GatedLinearAttention)
+register_part("mixer", "latent_attention", LatentAttention)
+register_part("feed_forward", "routed_experts", RoutedExperts)

@@ -19,7 +19,8 @@ from .base import Part
 
 
 class TokenEmbedding(Part):
-    """params: vocab_size, embed_dim (width of the table; projected to hidden if different)."""
+    """params: vocab_size, embed_dim (width of the table; projected to hidden if different), norm
+    (optional: the ``PartSpec`` of a norm applied to the embedded rows before the first layer)."""
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
@@ -28,19 +29,33 @@ class TokenEmbedding(Part):
         self.projected = self.embed_dim != hidden_size
         self.table = None
         self.w_in = None
+        self.norm = None
+        if spec.params.get("norm") is not None:
+            from .base import build_part
+            self.norm = build_part("norm", spec.params["norm"], hidden_size, dtype)
 
     def tensor_specs(self) -> List[TensorSpec]:
         specs = [TensorSpec(self.name("weight"), (self.vocab_size, self.embed_dim), "table")]
         if self.projected:
             specs.append(TensorSpec(self.name("project_in"), (self.hidden_size, self.embed_dim), "matrix"))
+        if self.norm is not None:
+            specs += self.norm.tensor_specs()
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.table = tensors[self.name("weight")]
         if self.projected:
             self.w_in = tensors[self.name("project_in")]
+        if self.norm is not None:
+            self.norm.bind(tensors)
 
     def forward(self, ctx, position) -> torch.Tensor:
+        x32 = self._embed(ctx, position)
+        if self.norm is not None:
+            _, x32 = self.norm.forward(x32, out_t=False, out_f32=True)
+        return x32
+
+    def _embed(self, ctx, position) -> torch.Tensor:
         T = ctx.num_tokens
         dev = self.table.device
         addend = position.embedding_addend(ctx) if position is not None else None

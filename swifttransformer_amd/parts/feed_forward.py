@@ -17,7 +17,8 @@ from .base import Part
 
 
 class DenseFeedForward(Part):
-    """params: inner (int), activation (a name the products' epilogues know), bias (bool)."""
+    """params: inner (int), activation (a name the products' epilogues know), bias (bool),
+    residual_scale (float, default 1: the factor with which the result enters the residual stream)."""
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
@@ -27,6 +28,7 @@ class DenseFeedForward(Part):
             raise ValueError(f"feed-forward activation {self.activation!r} has no kernel; "
                              f"available: {sorted(K.ACTIVATIONS)}")
         self.bias = bool(self.param("bias", True))
+        self.residual_scale = float(spec.params.get("residual_scale", 1.0))
         self.w1 = self.b1 = self.w2 = self.b2 = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -50,4 +52,4 @@ class DenseFeedForward(Part):
     def forward(self, x_t, residual32: torch.Tensor, ctx, norm=None) -> torch.Tensor:
         x_in = norm.as_input(residual32) if norm is not None else x_t
         h = K.gemm(x_in, self.w1, bias=self.b1, activation=self.activation)
-        return K.gemm(h, self.w2, bias=self.b2, residual=residual32, out_f32=True)
+        return K.gemm(h, self.w2, bias=self.b2, residual=residual32, out_f32=True, out_scale=self.residual_scale)

@@ -20,7 +20,8 @@ from .base import Part
 
 class LayerNorm(Part):
     """params: eps (float), affine (bool), center (bool, default True; False: root-mean-square norm),
-    bias (bool, default = affine: whether the affine part has a bias), width (int, default hidden_size)."""
+    bias (bool, default = affine: whether the affine part has a bias), width (int, default hidden_size),
+    scalar_gain (bool, default False: the file holds one number that multiplies every coordinate)."""
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
@@ -29,13 +30,14 @@ class LayerNorm(Part):
         self.center = bool(spec.params.get("center", True))
         self.has_bias = bool(spec.params.get("bias", self.affine)) and self.affine
         self.width = int(self.param("width", hidden_size))
+        self.scalar_gain = bool(spec.params.get("scalar_gain", False))
         self.gamma: Optional[torch.Tensor] = None
         self.beta: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
         if not self.affine:
             return []
-        specs = [TensorSpec(self.name("weight"), (self.width,), "vector", init="gain")]
+        specs = [TensorSpec(self.name("weight"), () if self.scalar_gain else (self.width,), "vector", init="gain")]
         if self.has_bias:
             specs.append(TensorSpec(self.name("bias"), (self.width,), "vector"))
         return specs
@@ -43,6 +45,8 @@ class LayerNorm(Part):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         if self.affine:
             self.gamma = tensors[self.name("weight")]
+            if self.scalar_gain:       # the kernels take a gain per coordinate
+                self.gamma = self.gamma.reshape(1).expand(self.width).contiguous()
             self.beta = tensors[self.name("bias")] if self.has_bias else None
 
     def fusable(self, rows: int, out_features: int) -> bool:

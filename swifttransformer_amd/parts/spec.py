@@ -24,6 +24,7 @@ class LayerSpec:
     mixer: PartSpec
     ffn_norm: Optional[PartSpec]
     feed_forward: Optional[PartSpec]
+    mixer_conv: Optional[PartSpec] = None   # a short filter over time on what the mixer reads
 
 
 @dataclass
