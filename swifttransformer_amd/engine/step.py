@@ -346,17 +346,18 @@ class ModelRunner:
                                   self.max_pages_per_seq, self.cache_param.page_size, self.device,
                                   self.model.max_positions, planned, extra)
             buffers.fill(items, tables, planned)
-            # the run before the recording does this batch's own work (its keys and values are
-            # written again, with the same values, by the replay below)
+            # The run before the recording is this batch's step: it has moved the requests' state on
+            # (a recurrent mixer's, a convolution's) and left its result where every replay leaves
+            # it, so this batch is not replayed on top of it.
             rec = self._capture(buffers, tune=T_pad <= self.tune_up_to, layers_only=True)
             while len(self._recorded_general) >= self.max_recorded:
                 self._recorded_general.pop(next(iter(self._recorded_general)))
             self._recorded_general[key] = rec
         else:
             rec.buffers.fill(items, tables, planned)
-        rec.graph.replay()
+            rec.graph.replay()
         self.steps_run += 1
-        self.graph_replays += 1
+        self.graph_replays += 1              # steps served by a recording, its first batch included
         best = torch.empty((R,), dtype=torch.int32, device=self.device)
         with using_arena(self.arena, rec.arena_state):
             logits = self.model.forward_head(rec.logits, rec.buffers.ctx, rec.buffers.ctx.want_rows[:R], keep=True,
