@@ -208,6 +208,95 @@ def kernel_times(args) -> int:
     return 0
 
 
+def side_by_side(args, shape: str) -> int:
+    """Zitupel beside OPT at the same layer sizes (width, heads, feed-forward width of OPT
+    ``shape``; the same number of layers, 8 unless ``--layers`` says otherwise; random weights):
+    decode tokens/s at batch 1, 8 and 64 from 1,024-token prompts, a 2,048-token prefill, and for
+    both the per-kernel times of one decode step at batch ``--batch`` and of the prefill with their
+    fractions of the memory or matrix floor (unrecorded steps, event pairs around the calls).
+    Prints one JSON line of its own."""
+    import gc
+    import torch
+    from swifttransformer_amd.config.registry import hyper_param_by_name
+    from swifttransformer_amd.engine.engine import Engine, parse_dtype
+    from swifttransformer_amd.engine.step import StepEntry
+    from swifttransformer_amd.models import random_model
+    from swifttransformer_amd.ops.profile import KernelTimer
+    layers = args.layers if args.layers != MODEL["num_hidden_layers"] else 8
+    dt = parse_dtype(args.dtype)
+    batch = args.batch
+    out = {"shape": shape, "layers": layers, "dtype": args.dtype, "models": {}}
+    for family in ("zitupel", "opt"):
+        over = {"num_layers": layers} if family == "zitupel" else {"num_hidden_layers": layers}
+        hp = hyper_param_by_name(f"{family}_{shape}", **over)
+        model = random_model(hp, dt, 0, "cuda:0")
+        weights = sum(t.numel() * t.element_size() for p in model.all_parts() for t in vars(p).values()
+                      if isinstance(t, torch.Tensor))
+        pages = 66 * (CONTEXT // PAGE)
+        eng = Engine(model, dtype=dt, page_size=PAGE, num_pages=pages, max_seqs=64,
+                     max_batched_tokens=64 * PROMPT_LEN, prefill_chunk=2048)
+        V = model.vocab_size
+        res = {"weight_bytes": weights}
+        for b, k in ((1, 64), (8, 64), (64, 32)):
+            d, ran, n, _ = decode_run(eng, b, k, 4, V, seed=b)
+            res[f"decode_b{b}_tokens_per_s"] = round(n / d, 1)
+            res[f"decode_b{b}_ms_per_step"] = round(d / ran * 1e3, 4)
+        pt = prefill_run(eng, 2048, V)
+        res["prefill_2048_ms"] = round(pt * 1e3, 3)
+        res["prefill_2048_tokens_per_s"] = round(2048 / pt, 1)
+        # per-kernel times, unrecorded
+        runner = eng.runner
+        runner.use_graphs = False
+        toks = prompts(batch + 1, CONTEXT, V, 5)
+        ctx_len = 1536
+        for i in range(batch):
+            runner.admit(i)
+            runner.step([StepEntry(i, toks[i][:ctx_len], [])])
+
+        def cost(keys_read, pairs):
+            def nbytes(name, info):
+                if name in ("attention_rows", "attention_prefill"):
+                    return 2 * keys_read * info["kv_heads"] * info["head_dim"] * info["elem"]
+                return None
+
+            def flops(name, info):
+                if name in ("attention_rows", "attention_prefill"):
+                    return 4.0 * pairs * info["heads"] * info["head_dim"]
+                return None
+            return nbytes, flops
+
+        def timed(entries_of, reps, keys_read, pairs):
+            for k in range(2):
+                runner.step(entries_of(k))
+            with KernelTimer() as t:
+                for k in range(2, 2 + reps):
+                    runner.step(entries_of(k))
+            rows = t.summary(*cost(keys_read, pairs))
+            for r in rows:
+                r["calls"] //= reps
+                r["us_total"] = round(r["us_total"] / reps, 1)
+            return {"us_sum_of_calls": round(sum(r["us_total"] for r in rows), 1), "kernels": rows}
+
+        res[f"kernels_decode_b{batch}"] = timed(
+            lambda k: [StepEntry(i, [toks[i][ctx_len + k]], [0]) for i in range(batch)], 6,
+            batch * (ctx_len + 5), batch * (ctx_len + 5))
+        for i in range(batch):
+            runner.finish(i)
+
+        def prefill(k):
+            if runner.is_live("p"):
+                runner.finish("p")
+            runner.admit("p")
+            return [StepEntry("p", toks[batch], [CONTEXT - 1])]
+        res["kernels_prefill_2048"] = timed(prefill, 3, CONTEXT, CONTEXT * (CONTEXT + 1) / 2.0)
+        out["models"][family] = res
+        del eng, runner, model
+        gc.collect()
+        torch.cuda.empty_cache()
+    print(json.dumps({"side_by_side": out}))
+    return 0
+
+
 def attention_only(args) -> int:
     """The prompt attention kernel alone on the model's geometry (one 2,048-row prompt, keys and
     values of one layer), three calls: for counter runs under the profiler.  `--attention-algo`
@@ -484,8 +573,10 @@ def main() -> int:
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     ap.add_argument("--workload", default="decode-1.3b",
-                    choices=["decode-1.3b", "mixed-6.7b", "mixed-1.3b", "ttft", "decode-30b", "decode-family"],
-                    help="decode-1.3b is the contract's line; the others are the other model shapes")
+                    choices=["decode-1.3b", "mixed-6.7b", "mixed-1.3b", "ttft", "decode-30b", "decode-family",
+                             "zitupel-125m", "zitupel-1.3b", "zitupel-6.7b"],
+                    help="decode-1.3b is the contract's line; the others are the other model shapes; zitupel-<size>: "
+                         "the Zitupel architecture beside OPT at the same layer sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -508,6 +599,8 @@ def main() -> int:
         return decode_30b(args)
     if args.workload == "decode-family":
         return decode_family(args)
+    if args.workload.startswith("zitupel-"):
+        return side_by_side(args, args.workload.split("-", 1)[1])
     steps = min(args.steps, CONTEXT - PROMPT_LEN)
     elem = 2 if args.dtype == "bf16" else 4
     biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)

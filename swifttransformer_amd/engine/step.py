@@ -74,6 +74,12 @@ class ModelRunner:
         self.model = model
         self.device = torch.device(device)
         max_pages = cache_param.max_pages_per_seq or cache_param.pages_for(model.max_positions)
+        if (not cache_param.max_pages_per_seq and gpu_mem_fraction <= 0 and isinstance(cache_param.num_pages, int)
+                and not any(need.window > 0 for need in model.cache_needs().values())):
+            # a request never holds more pages than the pool has: block tables need be no wider (models
+            # without a limit of their own would otherwise size them for positions no pool could hold);
+            # not so with windows, where a table goes on past pages that were given back
+            max_pages = min(max_pages, cache_param.num_pages)
         self.max_pages_per_seq = max_pages
         self.use_graphs = bool(use_graphs) and model.graph_safe and self.device.type == "cuda"
         self.planners = model.step_planners()

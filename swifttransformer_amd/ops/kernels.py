@@ -757,6 +757,7 @@ def token_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx_a
 
 
 # ------------------------------------------------------ gated linear attention
+@_timed("decay_gate", lambda z, inv_tau: {"rows": z.shape[0], "width": z.shape[-1], "bytes": 8 * z.numel()})
 def decay_gate(z: torch.Tensor, inv_tau: float) -> torch.Tensor:
     """In place: z <- sigmoid(z) ** inv_tau (float), computed as exp(inv_tau * log sigmoid(z))."""
     _need(z, "z", torch.float32)
@@ -769,7 +770,9 @@ def _d_gla_scan(q, k, v, decay, state, ctx_arrays, heads, scale):
     kd, vd = q.shape[1] // heads, v.shape[1] // heads
     return {"rows": T, "heads": heads, "key_dim": kd, "value_dim": vd, "items": ctx_arrays[2].shape[0],
             "flops": 4 * T * heads * kd * vd,
-            "bytes": T * heads * ((2 * kd + vd) * q.element_size() + 4 * kd + 4 * vd)}
+            # operands and results of every row, and the items' states read and written once
+            "bytes": T * heads * ((2 * kd + vd) * q.element_size() + 4 * kd + 4 * vd) +
+                     8 * ctx_arrays[2].shape[0] * heads * kd * vd}
 
 
 @_timed("gla_scan", _d_gla_scan)
@@ -800,6 +803,8 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Ten
     return out
 
 
+@_timed("gated_head_norm", lambda o, gate, *a, **k: {"rows": o.shape[0], "width": o.shape[1],
+                                                     "bytes": o.numel() * (4 + 2 * gate.element_size())})
 def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, heads: int, eps: float,
                     out_dtype: torch.dtype) -> torch.Tensor:
     """out[t, h, :] = o[t, h, :] * rsqrt(mean(o[t, h, :]^2) + eps) * gain * silu(gate[t, h, :]).
@@ -818,6 +823,8 @@ def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, hea
 
 
 # ------------------------------------------------------------------ latent cache
+@_timed("latent_write", lambda cache, x, *a, **k: {"rows": x.shape[0], "width": x.shape[1],
+                                                   "bytes": x.numel() * (4 + cache.element_size())})
 def latent_write(cache: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: float, token_item: torch.Tensor,
                  positions: torch.Tensor, block_table: torch.Tensor) -> None:
     """Each row of x (float [T, rank], dense rows of any stride) is normalised to unit root mean

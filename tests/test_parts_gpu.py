@@ -126,7 +126,7 @@ def test_feed_forward_part(dtype):
     ref = res.double() + P.feed_forward(d.double(), w, "l", True)
     check(out, ref, dtype, "feed-forward")
     with pytest.raises(ValueError, match="activation"):
-        build_part("feed_forward", PartSpec("dense", {"inner": 8, "activation": "gelu"}, names), H, dtype)
+        build_part("feed_forward", PartSpec("dense", {"inner": 8, "activation": "mish"}, names), H, dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
