@@ -74,8 +74,9 @@ class ZitupelHyperParam:
             if kind == "gla":
                 if _need(m, "tau", f"{w}.mixer", _NUM) <= 0:
                     raise ConfigError(f"config.json: {w}.mixer.tau must be positive")
-                if m["dim"] > 256:
-                    raise ConfigError(f"{w}.mixer.dim: up to 256 key channels a head, got {m['dim']}")
+                if m["dim"] > 256 or m["vdim"] > 256:
+                    raise ConfigError(f"{w}.mixer: up to 256 key and 256 value channels a head, got dim {m['dim']} "
+                                      f"and vdim {m['vdim']}")
             else:
                 _need(m, "kv_rank", f"{w}.mixer", (int,), 1)
                 _need(m, "scale", f"{w}.mixer", _NUM)

@@ -113,13 +113,14 @@ int st_token_conv_state(float* state, const float* x, const int* item_len, const
 // a = sigmoid(z)^(inv_tau), in place over n floats.
 int st_decay_gate(float* z, int64_t n, float inv_tau, hipStream_t stream);
 // Per item and head, from the state S [key_dim, value_dim] of the item's slot and over its rows in
-// order: S = diag(a_t) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.  q, k, v:
-// rows of `dtype` with their strides in elements (head h at h * key_dim / h * value_dim); a: float
-// [T, heads * key_dim]; o: float [T, heads * value_dim]; state: float [slots, heads, key_dim, value_dim].
+// order: S = diag(a_t) S + k_t v_t^T with a_t = sigmoid(z_t)^(inv_tau), o_t = scale * S^T q_t; the
+// state is stored back.  q, k, v: rows of `dtype` with their strides in elements (head h at
+// h * key_dim / h * value_dim); z: float [T, heads * key_dim]; o: float [T, heads * value_dim];
+// state: float [slots, heads, key_dim, value_dim].
 int st_gla_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
-                const void* v, int64_t v_stride, const float* a, float* state,
+                const void* v, int64_t v_stride, const float* z, float* state,
                 const int* item_len, const int* item_tok_off, const int* item_slot, int num_items,
-                int heads, int key_dim, int value_dim, float scale, int dtype, hipStream_t stream);
+                int heads, int key_dim, int value_dim, float scale, float inv_tau, int dtype, hipStream_t stream);
 // out[t, h, j] = o[t, h, j] * rsqrt(mean_j o[t, h, :]^2 + eps) * gain[j] * silu(g[t, h, j]); g: rows
 // of `dtype` with stride g_stride; out: rows of `dtype`, dense.
 int st_gated_head_norm(void* out, const float* o, const void* g, int64_t g_stride, const float* gain,
@@ -138,21 +139,22 @@ int st_latent_write(void* cache, int64_t page_stride, const float* x, int64_t x_
 // the lower index on ties, and sigmoid of their logits.  Rows whose item is -1 get ids of -1.
 int st_moe_route(int* ids, float* weights, const float* logits, const int* token_item, int num_tokens,
                  int experts, int top, hipStream_t stream);
-// Sorts the num_pairs = tokens * top (token, choice) pairs by expert into tiles of 16 entries that
-// hold one expert's pairs each: sorted[capacity] (pair index, or -1), place_of_pair[num_pairs]
-// (or -1), tile_expert[capacity / 16] (or -1).  capacity >= round_up(num_pairs, 16) + 16 * experts.
+// Sorts the num_pairs = tokens * top (token, choice) pairs by expert into tiles of `tile` (16 or 64)
+// places that hold one expert's pairs each: sorted[capacity] (pair index, or -1),
+// place_of_pair[num_pairs] (or -1), tile_expert[capacity / tile] (or -1).
+// capacity >= round_up(num_pairs, tile) + tile * experts.  The three calls below take the same `tile`.
 int st_moe_align(int* sorted, int* place_of_pair, int* tile_expert, const int* ids, int num_pairs,
-                 int experts, int capacity, hipStream_t stream);
+                 int experts, int capacity, int tile, hipStream_t stream);
 // y[place, f] = g * sigmoid(1.702 g) * (u + 1) with g = min(s * (x_t . Wg[e, f]), limit) and
 // u = clamp(s * (x_t . Wu[e, f]), -limit, limit), for the pair (t, j) at `place`, e its expert and s
 // its weight.  x: [T, width]; w_gate, w_up: [experts, inner, width]; y: [capacity, inner].
 int st_moe_up(void* y, const void* x, const void* w_gate, const void* w_up, const int* sorted,
-              const int* tile_expert, const float* weights, int capacity, int top, int width, int inner,
+              const int* tile_expert, const float* weights, int capacity, int tile, int top, int width, int inner,
               float limit, int dtype, hipStream_t stream);
 // pair_out[place, n] = y[place] . Wd[e, n] (top > 1), or, with top == 1, directly
 // out[t, n] = residual[t, n] + out_scale * y[place] . Wd[e, n].  w_down: [experts, width, inner].
 int st_moe_down(float* out, const float* residual, float* pair_out, const void* y, const void* w_down,
-                const int* sorted, const int* tile_expert, int capacity, int top, int width, int inner,
+                const int* sorted, const int* tile_expert, int capacity, int tile, int top, int width, int inner,
                 float out_scale, int dtype, hipStream_t stream);
 // out[t, n] = residual[t, n] + out_scale * sum_j pair_out[place_of_pair[t * top + j], n]
 int st_moe_combine(float* out, const float* residual, const float* pair_out, const int* place_of_pair,

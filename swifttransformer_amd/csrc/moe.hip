@@ -3,8 +3,8 @@
 //
 // Everything stays on the device and has a fixed launch shape, so a step can be recorded:
 //   route    per token the `top` largest router logits and the sigmoid of each;
-//   align    the (token, choice) pairs sorted by expert into tiles of 16 places, a tile holding
-//            pairs of one expert only (places left over are marked -1);
+//   align    the (token, choice) pairs sorted by expert into tiles of 16 or 64 places, a tile
+//            holding pairs of one expert only (places left over are marked -1);
 //   up       per tile and 64 inner features: both input products on the matrix cores, rows
 //            gathered through the sorted list, then clamp, gate and product of the two halves;
 //   down     per tile and 64 output features: the output product; with one expert a token the
@@ -21,7 +21,7 @@ namespace st {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kTile = 16;
+constexpr int kRows = 16;            // rows of one matrix-instruction block
 constexpr int kMaxTop = 16;
 
 __global__ __launch_bounds__(256) void moe_route_kernel(
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
 // gets depends on the order of the atomics; a pair's result does not depend on its place.
 __global__ __launch_bounds__(1024) void moe_align_kernel(
     int* __restrict__ sorted, int* __restrict__ place_of_pair, int* __restrict__ tile_expert,
-    const int* __restrict__ ids, int num_pairs, int experts, int capacity) {
+    const int* __restrict__ ids, int num_pairs, int experts, int capacity, int kTile) {
     extern __shared__ int lds[];
     int* count = lds;                  // [experts]
     int* offset = lds + experts;       // [experts + 1]
@@ -134,9 +134,11 @@ template <> struct Frag<float> {
     }
 };
 
-// grid (tiles, ceil(inner / 64)); wave w of the workgroup takes inner features f0 + 16 w .. +15.
-// Result layout of a wave: lane (r16, g) holds rows 4g .. 4g+3 of feature r16.
-template <typename T>
+// grid (tiles, ceil(inner / 64)); wave w of the workgroup takes inner features f0 + 16 w .. +15 of
+// the tile's RT blocks of 16 rows: a step's weight operands are loaded once and meet RT blocks of
+// rows (RT = 1 for few rows an expert, where only the weights' stream counts; RT = 4 for prompts).
+// Result layout of a block: lane (r16, g) holds rows 4g .. 4g+3 of feature r16.
+template <typename T, int RT>
 __global__ __launch_bounds__(256) void moe_up_kernel(
     T* __restrict__ y, const T* __restrict__ x, const T* __restrict__ w_gate, const T* __restrict__ w_up,
     const int* __restrict__ sorted, const int* __restrict__ tile_expert, const float* __restrict__ weights,
@@ -147,40 +149,55 @@ __global__ __launch_bounds__(256) void moe_up_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
     const int f = blockIdx.y * 64 + wave * 16 + r16;           // this lane's feature as an operand row
     const bool f_ok = f < inner;
-    const int pair = sorted[tile * kTile + r16];               // this lane's token row as an operand row
-    const bool p_ok = pair >= 0;
-    const T* xr = x + (int64_t)(p_ok ? pair / top : 0) * width;
+    const int base = tile * (kRows * RT);
+    const T* xr[RT];
+    bool p_ok[RT];
+#pragma unroll
+    for (int b = 0; b < RT; ++b) {
+        const int pair = sorted[base + b * kRows + r16];       // this lane's token row as an operand row
+        p_ok[b] = pair >= 0;
+        xr[b] = x + (int64_t)(p_ok[b] ? pair / top : 0) * width;
+    }
     const T* gr = w_gate + ((int64_t)e * inner + (f_ok ? f : 0)) * width;
     const T* ur = w_up + ((int64_t)e * inner + (f_ok ? f : 0)) * width;
-    floatx4 cg = {0.f, 0.f, 0.f, 0.f}, cu = {0.f, 0.f, 0.f, 0.f};
+    floatx4 cg[RT], cu[RT];
+#pragma unroll
+    for (int b = 0; b < RT; ++b) { cg[b] = floatx4{0.f, 0.f, 0.f, 0.f}; cu[b] = floatx4{0.f, 0.f, 0.f, 0.f}; }
     constexpr int D = Frag<T>::kDepth, L = Frag<T>::kLane;
+#pragma unroll 2
     for (int k0 = 0; k0 < width; k0 += D) {
-        Frag<T> a, bg, bu;
+        Frag<T> a[RT], bg, bu;
         const int k = k0 + L * g;
-        a.load(xr, k, width, p_ok, vec);
         bg.load(gr, k, width, f_ok, vec);
         bu.load(ur, k, width, f_ok, vec);
-        cg = Frag<T>::mma(a, bg, cg);
-        cu = Frag<T>::mma(a, bu, cu);
+#pragma unroll
+        for (int b = 0; b < RT; ++b) a[b].load(xr[b], k, width, p_ok[b], vec);
+#pragma unroll
+        for (int b = 0; b < RT; ++b) {
+            cg[b] = Frag<T>::mma(a[b], bg, cg[b]);
+            cu[b] = Frag<T>::mma(a[b], bu, cu[b]);
+        }
     }
     if (!f_ok) return;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int place = tile * kTile + 4 * g + r;
-        const int p = sorted[place];
-        float out = 0.f;
-        if (p >= 0) {
-            const float s = weights[p];
-            const float gv = fminf(s * cg[r], limit);
-            const float uv = fminf(fmaxf(s * cu[r], -limit), limit);
-            out = gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f);
+    for (int b = 0; b < RT; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int place = base + b * kRows + 4 * g + r;
+            const int p = sorted[place];
+            float out = 0.f;
+            if (p >= 0) {
+                const float s = weights[p];
+                const float gv = fminf(s * cg[b][r], limit);
+                const float uv = fminf(fmaxf(s * cu[b][r], -limit), limit);
+                out = gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f);
+            }
+            Elem<T>::store(y + (int64_t)place * inner + f, out);
         }
-        Elem<T>::store(y + (int64_t)place * inner + f, out);
-    }
 }
 
 // grid (tiles, ceil(width / 64)).
-template <typename T>
+template <typename T, int RT>
 __global__ __launch_bounds__(256) void moe_down_kernel(
     float* __restrict__ out, const float* __restrict__ residual, float* __restrict__ pair_out,
     const T* __restrict__ y, const T* __restrict__ w_down, const int* __restrict__ sorted,
@@ -191,30 +208,38 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
     const int n = blockIdx.y * 64 + wave * 16 + r16;
     const bool n_ok = n < width;
-    const T* yr = y + (int64_t)(tile * kTile + r16) * inner;
+    const int base = tile * (kRows * RT);
+    const T* yr = y + (int64_t)(base + r16) * inner;
     const T* wr = w_down + ((int64_t)e * width + (n_ok ? n : 0)) * inner;
-    floatx4 c = {0.f, 0.f, 0.f, 0.f};
+    floatx4 c[RT];
+#pragma unroll
+    for (int b = 0; b < RT; ++b) c[b] = floatx4{0.f, 0.f, 0.f, 0.f};
     constexpr int D = Frag<T>::kDepth, L = Frag<T>::kLane;
+#pragma unroll 2
     for (int k0 = 0; k0 < inner; k0 += D) {
-        Frag<T> a, b;
+        Frag<T> a[RT], bw;
         const int k = k0 + L * g;
-        a.load(yr, k, inner, true, vec);
-        b.load(wr, k, inner, n_ok, vec);
-        c = Frag<T>::mma(a, b, c);
+        bw.load(wr, k, inner, n_ok, vec);
+#pragma unroll
+        for (int b = 0; b < RT; ++b) a[b].load(yr + (int64_t)b * kRows * inner, k, inner, true, vec);
+#pragma unroll
+        for (int b = 0; b < RT; ++b) c[b] = Frag<T>::mma(a[b], bw, c[b]);
     }
     if (!n_ok) return;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int place = tile * kTile + 4 * g + r;
-        const int p = sorted[place];
-        if (p < 0) continue;
-        if (pair_out) {
-            pair_out[(int64_t)place * width + n] = c[r];
-        } else {                                               // one expert a token: p is the token
-            const int64_t at = (int64_t)p * width + n;
-            out[at] = fmaf(out_scale, c[r], residual[at]);
+    for (int b = 0; b < RT; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int place = base + b * kRows + 4 * g + r;
+            const int p = sorted[place];
+            if (p < 0) continue;
+            if (pair_out) {
+                pair_out[(int64_t)place * width + n] = c[b][r];
+            } else {                                           // one expert a token: p is the token
+                const int64_t at = (int64_t)p * width + n;
+                out[at] = fmaf(out_scale, c[b][r], residual[at]);
+            }
         }
-    }
 }
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(
@@ -252,13 +277,15 @@ extern "C" int st_moe_route(int* ids, float* weights, const float* logits, const
 }
 
 extern "C" int st_moe_align(int* sorted, int* place_of_pair, int* tile_expert, const int* ids, int num_pairs,
-                            int experts, int capacity, hipStream_t stream) {
+                            int experts, int capacity, int tile, hipStream_t stream) {
+    const int kTile = tile;
     ST_CHECK(num_pairs >= 0 && experts > 0 && experts <= 4096, "moe_align: bad sizes (up to 4096 experts)");
+    ST_CHECK(tile == 16 || tile == 64, "moe_align: tiles of 16 or 64 places, not %d", tile);
     ST_CHECK(capacity % kTile == 0 && capacity >= (num_pairs + kTile - 1) / kTile * kTile + kTile * experts,
              "moe_align: %d places do not hold %d pairs of %d experts in tiles of %d", capacity, num_pairs, experts, kTile);
     ST_CHECK(sorted && place_of_pair && tile_expert && ids, "moe_align: null operand");
     moe_align_kernel<<<1, 1024, (2 * experts + 1) * sizeof(int), stream>>>(sorted, place_of_pair, tile_expert, ids,
-                                                                          num_pairs, experts, capacity);
+                                                                          num_pairs, experts, capacity, tile);
     ST_LAUNCH_CHECK("moe_align");
     return 0;
 }
@@ -270,27 +297,31 @@ static bool rows_vectorised(const void* a, const void* b, const void* c, int dep
 }
 
 extern "C" int st_moe_up(void* y, const void* x, const void* w_gate, const void* w_up, const int* sorted,
-                         const int* tile_expert, const float* weights, int capacity, int top, int width, int inner,
-                         float limit, int dtype, hipStream_t stream) {
+                         const int* tile_expert, const float* weights, int capacity, int tile, int top, int width,
+                         int inner, float limit, int dtype, hipStream_t stream) {
+    const int kTile = tile;
+    ST_CHECK(tile == 16 || tile == 64, "moe_up: tiles of 16 or 64 places, not %d", tile);
     ST_CHECK(capacity > 0 && capacity % kTile == 0 && top >= 1 && width > 0 && inner > 0, "moe_up: bad sizes");
     ST_CHECK(y && x && w_gate && w_up && sorted && tile_expert && weights, "moe_up: null operand");
     const dim3 grid(capacity / kTile, (inner + 63) / 64);
     ST_CHECK(grid.y <= 65535, "moe_up: too many inner features");
     const int vec = rows_vectorised(x, w_gate, w_up, width, dtype);
-    if (dtype == kF32)
-        moe_up_kernel<float><<<grid, 256, 0, stream>>>((float*)y, (const float*)x, (const float*)w_gate,
-            (const float*)w_up, sorted, tile_expert, weights, top, width, inner, limit, vec);
-    else if (dtype == kBF16)
-        moe_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)y, (const bf16_t*)x, (const bf16_t*)w_gate,
-            (const bf16_t*)w_up, sorted, tile_expert, weights, top, width, inner, limit, vec);
+#define ST_UP(T, RT)                                                                                         \
+    moe_up_kernel<T, RT><<<grid, 256, 0, stream>>>((T*)y, (const T*)x, (const T*)w_gate, (const T*)w_up, sorted, \
+                                                   tile_expert, weights, top, width, inner, limit, vec)
+    if (dtype == kF32) { if (tile == 16) ST_UP(float, 1); else ST_UP(float, 4); }
+    else if (dtype == kBF16) { if (tile == 16) ST_UP(bf16_t, 1); else ST_UP(bf16_t, 4); }
     else ST_CHECK(false, "moe_up: unknown dtype %d", dtype);
+#undef ST_UP
     ST_LAUNCH_CHECK("moe_up");
     return 0;
 }
 
 extern "C" int st_moe_down(float* out, const float* residual, float* pair_out, const void* y, const void* w_down,
-                           const int* sorted, const int* tile_expert, int capacity, int top, int width, int inner,
-                           float out_scale, int dtype, hipStream_t stream) {
+                           const int* sorted, const int* tile_expert, int capacity, int tile, int top, int width,
+                           int inner, float out_scale, int dtype, hipStream_t stream) {
+    const int kTile = tile;
+    ST_CHECK(tile == 16 || tile == 64, "moe_down: tiles of 16 or 64 places, not %d", tile);
     ST_CHECK(capacity > 0 && capacity % kTile == 0 && top >= 1 && width > 0 && inner > 0, "moe_down: bad sizes");
     ST_CHECK(y && w_down && sorted && tile_expert, "moe_down: null operand");
     ST_CHECK(pair_out ? true : (top == 1 && out && residual),
@@ -298,13 +329,13 @@ extern "C" int st_moe_down(float* out, const float* residual, float* pair_out, c
     const dim3 grid(capacity / kTile, (width + 63) / 64);
     ST_CHECK(grid.y <= 65535, "moe_down: too wide");
     const int vec = rows_vectorised(y, w_down, w_down, inner, dtype);
-    if (dtype == kF32)
-        moe_down_kernel<float><<<grid, 256, 0, stream>>>(out, residual, pair_out, (const float*)y, (const float*)w_down,
-            sorted, tile_expert, top, width, inner, out_scale, vec);
-    else if (dtype == kBF16)
-        moe_down_kernel<bf16_t><<<grid, 256, 0, stream>>>(out, residual, pair_out, (const bf16_t*)y,
-            (const bf16_t*)w_down, sorted, tile_expert, top, width, inner, out_scale, vec);
+#define ST_DOWN(T, RT)                                                                                        \
+    moe_down_kernel<T, RT><<<grid, 256, 0, stream>>>(out, residual, pair_out, (const T*)y, (const T*)w_down,      \
+                                                     sorted, tile_expert, top, width, inner, out_scale, vec)
+    if (dtype == kF32) { if (tile == 16) ST_DOWN(float, 1); else ST_DOWN(float, 4); }
+    else if (dtype == kBF16) { if (tile == 16) ST_DOWN(bf16_t, 1); else ST_DOWN(bf16_t, 4); }
     else ST_CHECK(false, "moe_down: unknown dtype %d", dtype);
+#undef ST_DOWN
     ST_LAUNCH_CHECK("moe_down");
     return 0;
 }

@@ -70,16 +70,16 @@ def _lib():
         lib.st_token_conv_state.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
         lib.st_decay_gate.argtypes = [_c_p, _c_i64, _c_f, _c_p]
         lib.st_gla_scan.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p,
-                                    _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
+                                    _c_int, _c_int, _c_int, _c_int, _c_f, _c_f, _c_int, _c_p]
         lib.st_gated_head_norm.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
         lib.st_latent_write.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
                                         _c_int, _c_int, _c_f, _c_int, _c_p]
         lib.st_moe_route.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
-        lib.st_moe_align.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
-        lib.st_moe_up.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_f,
-                                  _c_int, _c_p]
-        lib.st_moe_down.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_f,
-                                    _c_int, _c_p]
+        lib.st_moe_align.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_p]
+        lib.st_moe_up.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                  _c_f, _c_int, _c_p]
+        lib.st_moe_down.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                    _c_f, _c_int, _c_p]
         lib.st_moe_combine.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_f, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
@@ -765,7 +765,7 @@ def decay_gate(z: torch.Tensor, inv_tau: float) -> torch.Tensor:
     return z
 
 
-def _d_gla_scan(q, k, v, decay, state, ctx_arrays, heads, scale):
+def _d_gla_scan(q, k, v, gate, state, ctx_arrays, heads, scale, inv_tau):
     T = q.shape[0]
     kd, vd = q.shape[1] // heads, v.shape[1] // heads
     return {"rows": T, "heads": heads, "key_dim": kd, "value_dim": vd, "items": ctx_arrays[2].shape[0],
@@ -776,13 +776,14 @@ def _d_gla_scan(q, k, v, decay, state, ctx_arrays, heads, scale):
 
 
 @_timed("gla_scan", _d_gla_scan)
-def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
-             ctx_arrays, heads: int, scale: float) -> torch.Tensor:
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor, state: torch.Tensor,
+             ctx_arrays, heads: int, scale: float, inv_tau: float) -> torch.Tensor:
     """Per item and head, from the slot's state S and over the item's rows in order:
-    S <- diag(decay_t) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.
+    S <- diag(a_t) S + k_t v_t^T with the decay a_t = sigmoid(gate_t) ** inv_tau, o_t = scale * S^T q_t;
+    the state is stored back.
 
     q, k: [T, heads * key_dim], v: [T, heads * value_dim] views (dense rows, any row stride);
-    decay: float [T, heads * key_dim]; state: float [slots, heads, key_dim, value_dim].  Returns
+    gate: float [T, heads * key_dim]; state: float [slots, heads, key_dim, value_dim].  Returns
     float [T, heads * value_dim]."""
     _token_item, item_len, item_tok_off, item_slot = ctx_arrays
     T = q.shape[0]
@@ -791,15 +792,15 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Ten
         _need(t, name, q.dtype, (T, w), contiguous=False)
         if t.stride(1) != 1:
             raise KernelError(f"{name}: rows must be dense")
-    _need(decay, "decay", torch.float32, (T, heads * kd))
+    _need(gate, "gate", torch.float32, (T, heads * kd))
     _need(state, "state", torch.float32, (state.shape[0], heads, kd, vd))
     B = item_slot.shape[0]
     for name, t in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
         _need(t, name, torch.int32, (B,))
     out = empty((T, heads * vd), torch.float32, q.device)
     _check(_lib().st_gla_scan(_ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
-                              _ptr(decay), _ptr(state), _ptr(item_len), _ptr(item_tok_off), _ptr(item_slot), B,
-                              heads, kd, vd, float(scale), dtype_code(q.dtype), _stream()))
+                              _ptr(gate), _ptr(state), _ptr(item_len), _ptr(item_tok_off), _ptr(item_slot), B,
+                              heads, kd, vd, float(scale), float(inv_tau), dtype_code(q.dtype), _stream()))
     return out
 
 
@@ -848,12 +849,15 @@ def latent_write(cache: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: 
 
 
 # ---------------------------------------------------------------- routed experts
-MOE_TILE = 16
+def moe_tile(num_tokens: int, top: int, experts: int) -> int:
+    """Places a tile: 64 where an expert gets some dozens of rows on average (a tile's weight
+    operands then meet four blocks of 16 rows), else 16 (few rows: only the weights' stream counts)."""
+    return 64 if num_tokens * top >= 32 * experts else 16
 
 
-def moe_capacity(num_tokens: int, top: int, experts: int) -> int:
+def moe_capacity(num_tokens: int, top: int, experts: int, tile: int) -> int:
     """Places of the sorted pair list: every expert's pairs start a tile of their own."""
-    return -(-num_tokens * top // MOE_TILE) * MOE_TILE + MOE_TILE * experts
+    return -(-num_tokens * top // tile) * tile + tile * experts
 
 
 def _d_moe(x, logits, w_gate, w_up, w_down, residual, *, top, limit, out_scale=1.0, token_item=None):
@@ -886,24 +890,25 @@ def routed_experts(x: torch.Tensor, logits: torch.Tensor, w_gate: torch.Tensor, 
     if token_item is not None:
         _need(token_item, "token_item", torch.int32, (T,))
     lib, dev, code, st = _lib(), x.device, dtype_code(x.dtype), _stream()
-    cap = moe_capacity(T, top, E)
+    tile = moe_tile(T, top, E)
+    cap = moe_capacity(T, top, E, tile)
     ids = empty((T * top,), torch.int32, dev)
     wts = empty((T * top,), torch.float32, dev)
     sorted_pairs = empty((cap,), torch.int32, dev)
     place = empty((T * top,), torch.int32, dev)
-    tile_expert = empty((cap // MOE_TILE,), torch.int32, dev)
+    tile_expert = empty((cap // tile,), torch.int32, dev)
     y = empty((cap, F), x.dtype, dev)
     _check(lib.st_moe_route(_ptr(ids), _ptr(wts), _ptr(logits), _ptr(token_item), T, E, int(top), st))
-    _check(lib.st_moe_align(_ptr(sorted_pairs), _ptr(place), _ptr(tile_expert), _ptr(ids), T * top, E, cap, st))
+    _check(lib.st_moe_align(_ptr(sorted_pairs), _ptr(place), _ptr(tile_expert), _ptr(ids), T * top, E, cap, tile, st))
     _check(lib.st_moe_up(_ptr(y), _ptr(x), _ptr(w_gate), _ptr(w_up), _ptr(sorted_pairs), _ptr(tile_expert),
-                         _ptr(wts), cap, int(top), W, F, float(limit), code, st))
+                         _ptr(wts), cap, tile, int(top), W, F, float(limit), code, st))
     if top == 1:
         _check(lib.st_moe_down(_ptr(residual), _ptr(residual), None, _ptr(y), _ptr(w_down), _ptr(sorted_pairs),
-                               _ptr(tile_expert), cap, 1, W, F, float(out_scale), code, st))
+                               _ptr(tile_expert), cap, tile, 1, W, F, float(out_scale), code, st))
     else:
         pair_out = empty((cap, W), torch.float32, dev)
         _check(lib.st_moe_down(None, None, _ptr(pair_out), _ptr(y), _ptr(w_down), _ptr(sorted_pairs),
-                               _ptr(tile_expert), cap, int(top), W, F, float(out_scale), code, st))
+                               _ptr(tile_expert), cap, tile, int(top), W, F, float(out_scale), code, st))
         _check(lib.st_moe_combine(_ptr(residual), _ptr(residual), _ptr(pair_out), _ptr(place), T, int(top), W,
                                   float(out_scale), st))
     return residual

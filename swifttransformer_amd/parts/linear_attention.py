@@ -37,8 +37,9 @@ class GatedLinearAttention(Mixer):
         self.residual_scale = float(spec.params.get("residual_scale", 1.0))
         if self.tau <= 0:
             raise ValueError(f"tau must be positive, got {self.tau}")
-        if self.key_dim > 256:
-            raise ValueError(f"the scan kernel takes up to 256 key channels a head, not {self.key_dim}")
+        if self.key_dim > 256 or self.value_dim > 256:
+            raise ValueError(f"the scan kernel takes up to 256 key and 256 value channels a head, not "
+                             f"{self.key_dim} and {self.value_dim}")
         self.qk_size = self.num_heads * self.key_dim
         self.v_size = self.num_heads * self.value_dim
         self.scale = float(self.key_dim) ** -0.5
@@ -72,9 +73,9 @@ class GatedLinearAttention(Mixer):
         qk, vs = self.qk_size, self.v_size
         proj = K.gemm(x_t, self.w_in)
         low = K.gemm(x_t, self.w_decay_in)
-        decay = K.decay_gate(K.gemm(low, self.w_decay_out, bias=self.b_decay, out_f32=True), 1.0 / self.tau)
+        gate = K.gemm(low, self.w_decay_out, bias=self.b_decay, out_f32=True)      # the decay's logits, float
         items = (ctx.token_item, ctx.item_len, ctx.item_tok_off, ctx.item_slot)
-        o = K.gla_scan(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + vs], decay, cache.state, items,
-                       self.num_heads, self.scale)
+        o = K.gla_scan(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + vs], gate, cache.state, items,
+                       self.num_heads, self.scale, 1.0 / self.tau)
         y = K.gated_head_norm(o, proj[:, 2 * qk + vs:], self.gain, self.num_heads, self.eps, self.dtype)
         return K.gemm(y, self.w_out, residual=residual32, out_f32=True, out_scale=self.residual_scale)

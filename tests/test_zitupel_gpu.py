@@ -113,9 +113,9 @@ def test_gla_scan_whole_portions_and_single_tokens(dtype, heads, kd, vd):
     rnd = lambda *s: torch.randn(*s, generator=g).to(dt).to(F64)        # values the storage type holds
     q, k, v = rnd(T, heads, kd), rnd(T, heads, kd) * 0.5, rnd(T, heads, vd)
     z = torch.randn(T, heads * kd, generator=g) * 2 + 1
-    decay = K.decay_gate(dev(z), 1 / 3.0)
     a = torch.sigmoid(z.to(F64)).pow(1 / 3.0)
-    check(decay, a.numpy(), torch.float32, "decay gate")
+    check(K.decay_gate(dev(z), 1 / 3.0), a.numpy(), torch.float32, "decay gate")
+    decay = dev(z)                                                       # the scan takes the logits
     want, S_end = plain_scan(q, k, v, a.view(T, heads, kd), torch.zeros(heads, kd, vd, dtype=F64), 0.37)
     # one fused row [q | junk | k | v] so that the operands are strided views
     fused = torch.cat([q.reshape(T, -1), torch.full((T, 8), float("nan"), dtype=F64), k.reshape(T, -1), v.reshape(T, -1)], 1)
@@ -128,7 +128,7 @@ def test_gla_scan_whole_portions_and_single_tokens(dtype, heads, kd, vd):
         for n in cuts:
             rows = fused[lo:lo + n]
             got.append(K.gla_scan(rows[:, :o0], rows[:, o1:o2], rows[:, o2:], decay[lo:lo + n], state,
-                                  items_ctx([n], [1]), heads, 0.37))
+                                  items_ctx([n], [1]), heads, 0.37, 1 / 3.0))
             lo += n
         what = f"{dtype} heads {heads} key {kd} value {vd} cuts {cuts[:4]}"
         check(torch.cat(got), want.reshape(T, -1).numpy(), torch.float32 if dt == torch.float32 else dt, what)
@@ -137,7 +137,7 @@ def test_gla_scan_whole_portions_and_single_tokens(dtype, heads, kd, vd):
     # two items in one launch, the second a padding item
     state = torch.zeros((2, heads, kd, vd), device=DEV)
     ti, ln, off, sl = items_ctx([T, 0], [0, -1])
-    got = K.gla_scan(fused[:, :o0], fused[:, o1:o2], fused[:, o2:], decay, state, (ti, ln, off, sl), heads, 0.37)
+    got = K.gla_scan(fused[:, :o0], fused[:, o1:o2], fused[:, o2:], decay, state, (ti, ln, off, sl), heads, 0.37, 1 / 3.0)
     check(got, want.reshape(T, -1).numpy(), torch.float32 if dt == torch.float32 else dt, "with a padding item")
 
 
