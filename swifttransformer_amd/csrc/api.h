@@ -139,7 +139,7 @@ int st_latent_write(void* cache, int64_t page_stride, const float* x, int64_t x_
 // the lower index on ties, and sigmoid of their logits.  Rows whose item is -1 get ids of -1.
 int st_moe_route(int* ids, float* weights, const float* logits, const int* token_item, int num_tokens,
                  int experts, int top, hipStream_t stream);
-// Sorts the num_pairs = tokens * top (token, choice) pairs by expert into tiles of `tile` (16 or 64)
+// Sorts the num_pairs = tokens * top (token, choice) pairs by expert into tiles of `tile` (16, 64 or 128)
 // places that hold one expert's pairs each: sorted[capacity] (pair index, or -1),
 // place_of_pair[num_pairs] (or -1), tile_expert[capacity / tile] (or -1).
 // capacity >= round_up(num_pairs, tile) + tile * experts.  The three calls below take the same `tile`.

@@ -3,7 +3,7 @@
 //
 // Everything stays on the device and has a fixed launch shape, so a step can be recorded:
 //   route    per token the `top` largest router logits and the sigmoid of each;
-//   align    the (token, choice) pairs sorted by expert into tiles of 16 or 64 places, a tile
+//   align    the (token, choice) pairs sorted by expert into tiles of 16, 64 or 128 places, a tile
 //            holding pairs of one expert only (places left over are marked -1);
 //   up       per tile and 64 inner features: both input products on the matrix cores, rows
 //            gathered through the sorted list, then clamp, gate and product of the two halves;
@@ -136,7 +136,8 @@ template <> struct Frag<float> {
 
 // grid (tiles, ceil(inner / 64)); wave w of the workgroup takes inner features f0 + 16 w .. +15 of
 // the tile's RT blocks of 16 rows: a step's weight operands are loaded once and meet RT blocks of
-// rows (RT = 1 for few rows an expert, where only the weights' stream counts; RT = 4 for prompts).
+// rows (RT = 1 for few rows an expert, where only the weights' stream counts; RT = 4 or 8 for
+// prompts, where every tile reads its expert's weights again from the L2).
 // Result layout of a block: lane (r16, g) holds rows 4g .. 4g+3 of feature r16.
 template <typename T, int RT>
 __global__ __launch_bounds__(256) void moe_up_kernel(
@@ -164,7 +165,7 @@ __global__ __launch_bounds__(256) void moe_up_kernel(
 #pragma unroll
     for (int b = 0; b < RT; ++b) { cg[b] = floatx4{0.f, 0.f, 0.f, 0.f}; cu[b] = floatx4{0.f, 0.f, 0.f, 0.f}; }
     constexpr int D = Frag<T>::kDepth, L = Frag<T>::kLane;
-#pragma unroll 2
+
     for (int k0 = 0; k0 < width; k0 += D) {
         Frag<T> a[RT], bg, bu;
         const int k = k0 + L * g;
@@ -215,7 +216,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
 #pragma unroll
     for (int b = 0; b < RT; ++b) c[b] = floatx4{0.f, 0.f, 0.f, 0.f};
     constexpr int D = Frag<T>::kDepth, L = Frag<T>::kLane;
-#pragma unroll 2
+
     for (int k0 = 0; k0 < inner; k0 += D) {
         Frag<T> a[RT], bw;
         const int k = k0 + L * g;
@@ -240,6 +241,141 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
                 out[at] = fmaf(out_scale, c[b][r], residual[at]);
             }
         }
+}
+
+// ---- prompts in bfloat16: tiles of 128 places, operands staged through LDS ----------------------
+// With a hundred rows and more an expert the products are bound by arithmetic, not by the weights'
+// stream, and operands read straight from memory leave the matrix cores waiting.  Here a workgroup
+// computes 128 places x 128 weight rows in steps of 64 in depth: all threads bring the two operand
+// tiles into registers with 16-byte loads (the next step's while this one is multiplied), store
+// them into LDS with the rows' chunks rotated so that the matrix instruction's reads spread over
+// the banks, and every wave multiplies a 64 x 64 part (v_mfma_f32_32x32x16_bf16).
+// UP: the 128 weight rows are 64 inner features of the gate matrix and the same 64 of the other
+// one, dealt so that a lane holds both halves of a result; rows of x are gathered through the
+// sorted list.  Otherwise: 128 output features of the expert's output matrix over the rows of y.
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+__device__ inline int rot(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
+
+template <bool UP>
+__global__ __launch_bounds__(256) void moe_tiled_kernel(
+    bf16_t* __restrict__ y_out, float* __restrict__ out, const float* __restrict__ residual,
+    float* __restrict__ pair_out, const bf16_t* __restrict__ a_rows, const bf16_t* __restrict__ w0,
+    const bf16_t* __restrict__ w1, const int* __restrict__ sorted, const int* __restrict__ tile_expert,
+    const float* __restrict__ weights, int top, int N, int K, float limit, float out_scale) {
+    __shared__ uint4 sw[128 * 8];      // weight rows: [row][chunk of 8 in depth]
+    __shared__ uint4 sx[128 * 8];      // places
+    const int tile = blockIdx.x;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wn = wave & 1, wm = wave >> 1, l32 = lane & 31, lh = lane >> 5;
+    const int base = tile * 128;
+    const int n0 = blockIdx.y * (UP ? 64 : 128);
+    // the four rows of each tile that this thread brings in, fixed over the steps
+    const bf16_t* wrow[4];
+    const bf16_t* xrow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = (tid + i * 256) >> 3;
+        int n;
+        const bf16_t* m;
+        if (UP) { n = n0 + (row >> 6) * 32 + (row & 31); m = ((row >> 5) & 1) ? w1 : w0; }
+        else { n = n0 + row; m = w0; }
+        wrow[i] = n < N ? m + ((int64_t)e * N + n) * K : nullptr;
+        const int p = sorted[base + row];
+        xrow[i] = UP ? (p >= 0 ? a_rows + (int64_t)(p / top) * K : nullptr) : a_rows + (int64_t)(base + row) * K;
+    }
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+    uint4 rw[4], rx[4];
+    auto load_global = [&](int k0) {
+        const int k = k0 + (tid & 7) * 8;
+        const bool in = k < K;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // (addresses clamped and values cleared rather than loads behind a branch)
+            const bf16_t* pw = wrow[i] ? wrow[i] : w0;
+            const bf16_t* px = xrow[i] ? xrow[i] : a_rows;
+            const uint4 vw = *reinterpret_cast<const uint4*>(pw + (in ? k : 0));
+            const uint4 vx = *reinterpret_cast<const uint4*>(px + (in ? k : 0));
+            rw[i] = (in && wrow[i]) ? vw : make_uint4(0, 0, 0, 0);
+            rx[i] = (in && xrow[i]) ? vx : make_uint4(0, 0, 0, 0);
+        }
+    };
+    load_global(0);
+    for (int k0 = 0; k0 < K; k0 += 64) {
+        __syncthreads();               // the step before has been read
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + i * 256;
+            sw[rot(c >> 3, c & 7)] = rw[i];
+            sx[rot(c >> 3, c & 7)] = rx[i];
+        }
+        __syncthreads();
+        if (k0 + 64 < K) load_global(k0 + 64);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            const int chunk = kk * 2 + lh;
+            bf16x8 a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = __builtin_bit_cast(bf16x8, sw[rot(wn * 64 + i * 32 + l32, chunk)]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = __builtin_bit_cast(bf16x8, sx[rot(wm * 64 + j * 32 + l32, chunk)]);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    // acc[i][j][q]: weight row wn*64 + i*32 + 8*(q/4) + 4*lh + q%4, place base + wm*64 + j*32 + l32
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int place = base + wm * 64 + j * 32 + l32;
+        const int p = sorted[place];
+        if (UP) {
+            const float s = p >= 0 ? weights[p] : 0.f;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int f = n0 + wn * 32 + 8 * q4 + 4 * lh;
+                if (f >= N) continue;
+                float r[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const float gv = fminf(s * acc[0][j][4 * q4 + u], limit);
+                    const float uv = fminf(fmaxf(s * acc[1][j][4 * q4 + u], -limit), limit);
+                    r[u] = p >= 0 ? gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f) : 0.f;
+                }
+                bf16_t* dst = y_out + (int64_t)place * N + f;
+                if (f + 3 < N && (N & 3) == 0) Elem<bf16_t>::store4(dst, r);
+                else
+                    for (int u = 0; u < 4 && f + u < N; ++u) Elem<bf16_t>::store(dst + u, r[u]);
+            }
+        } else {
+            if (p < 0) continue;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const int n = n0 + wn * 64 + i * 32 + 8 * q4 + 4 * lh;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (n + u >= N) continue;
+                        const float v = acc[i][j][4 * q4 + u];
+                        if (pair_out) pair_out[(int64_t)place * N + n + u] = v;
+                        else {
+                            const int64_t at = (int64_t)p * N + n + u;       // one expert a token: p is the token
+                            out[at] = fmaf(out_scale, v, residual[at]);
+                        }
+                    }
+                }
+        }
+    }
 }
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(
@@ -280,7 +416,7 @@ extern "C" int st_moe_align(int* sorted, int* place_of_pair, int* tile_expert, c
                             int experts, int capacity, int tile, hipStream_t stream) {
     const int kTile = tile;
     ST_CHECK(num_pairs >= 0 && experts > 0 && experts <= 4096, "moe_align: bad sizes (up to 4096 experts)");
-    ST_CHECK(tile == 16 || tile == 64, "moe_align: tiles of 16 or 64 places, not %d", tile);
+    ST_CHECK(tile == 16 || tile == 64 || tile == 128, "moe_align: tiles of 16, 64 or 128 places, not %d", tile);
     ST_CHECK(capacity % kTile == 0 && capacity >= (num_pairs + kTile - 1) / kTile * kTile + kTile * experts,
              "moe_align: %d places do not hold %d pairs of %d experts in tiles of %d", capacity, num_pairs, experts, kTile);
     ST_CHECK(sorted && place_of_pair && tile_expert && ids, "moe_align: null operand");
@@ -300,17 +436,24 @@ extern "C" int st_moe_up(void* y, const void* x, const void* w_gate, const void*
                          const int* tile_expert, const float* weights, int capacity, int tile, int top, int width,
                          int inner, float limit, int dtype, hipStream_t stream) {
     const int kTile = tile;
-    ST_CHECK(tile == 16 || tile == 64, "moe_up: tiles of 16 or 64 places, not %d", tile);
+    ST_CHECK(tile == 16 || tile == 64 || tile == 128, "moe_up: tiles of 16, 64 or 128 places, not %d", tile);
     ST_CHECK(capacity > 0 && capacity % kTile == 0 && top >= 1 && width > 0 && inner > 0, "moe_up: bad sizes");
     ST_CHECK(y && x && w_gate && w_up && sorted && tile_expert && weights, "moe_up: null operand");
     const dim3 grid(capacity / kTile, (inner + 63) / 64);
     ST_CHECK(grid.y <= 65535, "moe_up: too many inner features");
     const int vec = rows_vectorised(x, w_gate, w_up, width, dtype);
+    if (dtype == kBF16 && tile == 128 && vec) {
+        const dim3 g2(capacity / 128, (inner + 63) / 64);
+        moe_tiled_kernel<true><<<g2, 256, 0, stream>>>((bf16_t*)y, nullptr, nullptr, nullptr, (const bf16_t*)x,
+            (const bf16_t*)w_gate, (const bf16_t*)w_up, sorted, tile_expert, weights, top, inner, width, limit, 1.f);
+        ST_LAUNCH_CHECK("moe_up (tiled)");
+        return 0;
+    }
 #define ST_UP(T, RT)                                                                                         \
     moe_up_kernel<T, RT><<<grid, 256, 0, stream>>>((T*)y, (const T*)x, (const T*)w_gate, (const T*)w_up, sorted, \
                                                    tile_expert, weights, top, width, inner, limit, vec)
-    if (dtype == kF32) { if (tile == 16) ST_UP(float, 1); else ST_UP(float, 4); }
-    else if (dtype == kBF16) { if (tile == 16) ST_UP(bf16_t, 1); else ST_UP(bf16_t, 4); }
+    if (dtype == kF32) { if (tile == 16) ST_UP(float, 1); else if (tile == 64) ST_UP(float, 4); else ST_UP(float, 8); }
+    else if (dtype == kBF16) { if (tile == 16) ST_UP(bf16_t, 1); else if (tile == 64) ST_UP(bf16_t, 4); else ST_UP(bf16_t, 8); }
     else ST_CHECK(false, "moe_up: unknown dtype %d", dtype);
 #undef ST_UP
     ST_LAUNCH_CHECK("moe_up");
@@ -321,7 +464,7 @@ extern "C" int st_moe_down(float* out, const float* residual, float* pair_out, c
                            const int* sorted, const int* tile_expert, int capacity, int tile, int top, int width,
                            int inner, float out_scale, int dtype, hipStream_t stream) {
     const int kTile = tile;
-    ST_CHECK(tile == 16 || tile == 64, "moe_down: tiles of 16 or 64 places, not %d", tile);
+    ST_CHECK(tile == 16 || tile == 64 || tile == 128, "moe_down: tiles of 16, 64 or 128 places, not %d", tile);
     ST_CHECK(capacity > 0 && capacity % kTile == 0 && top >= 1 && width > 0 && inner > 0, "moe_down: bad sizes");
     ST_CHECK(y && w_down && sorted && tile_expert, "moe_down: null operand");
     ST_CHECK(pair_out ? true : (top == 1 && out && residual),
@@ -329,11 +472,18 @@ extern "C" int st_moe_down(float* out, const float* residual, float* pair_out, c
     const dim3 grid(capacity / kTile, (width + 63) / 64);
     ST_CHECK(grid.y <= 65535, "moe_down: too wide");
     const int vec = rows_vectorised(y, w_down, w_down, inner, dtype);
+    if (dtype == kBF16 && tile == 128 && vec) {
+        const dim3 g2(capacity / 128, (width + 127) / 128);
+        moe_tiled_kernel<false><<<g2, 256, 0, stream>>>(nullptr, out, residual, pair_out, (const bf16_t*)y,
+            (const bf16_t*)w_down, nullptr, sorted, tile_expert, nullptr, top, width, inner, 0.f, out_scale);
+        ST_LAUNCH_CHECK("moe_down (tiled)");
+        return 0;
+    }
 #define ST_DOWN(T, RT)                                                                                        \
     moe_down_kernel<T, RT><<<grid, 256, 0, stream>>>(out, residual, pair_out, (const T*)y, (const T*)w_down,      \
                                                      sorted, tile_expert, top, width, inner, out_scale, vec)
-    if (dtype == kF32) { if (tile == 16) ST_DOWN(float, 1); else ST_DOWN(float, 4); }
-    else if (dtype == kBF16) { if (tile == 16) ST_DOWN(bf16_t, 1); else ST_DOWN(bf16_t, 4); }
+    if (dtype == kF32) { if (tile == 16) ST_DOWN(float, 1); else if (tile == 64) ST_DOWN(float, 4); else ST_DOWN(float, 8); }
+    else if (dtype == kBF16) { if (tile == 16) ST_DOWN(bf16_t, 1); else if (tile == 64) ST_DOWN(bf16_t, 4); else ST_DOWN(bf16_t, 8); }
     else ST_CHECK(false, "moe_down: unknown dtype %d", dtype);
 #undef ST_DOWN
     ST_LAUNCH_CHECK("moe_down");

@@ -26,27 +26,33 @@ __global__ __launch_bounds__(256) void decay_gate_kernel(float* __restrict__ z, 
 
 // One workgroup per (item, head): wave w takes the value channels 16 w .. 16 w + 15, its four
 // 16-lane rows a quarter of the key channels each (DQ a lane, state in registers).  The item's
-// rows are walked in chunks: all threads together bring a chunk's q, k, decay logits and v from
-// memory into registers (every load in flight at once, while the chunk before is being
-// computed), then into LDS as floats, the decay a = exp(log sigmoid(z) / tau) computed on the way
-// once an element; then every lane reads what it needs from LDS, a token at a time.
-// LDS row of a token: q [KP] | k [KP] | a [KP] | v [VP], KP = 4 DQ >= key_dim and VP = 16 waves,
-// the padding zero (a padded key channel then adds nothing).  J: columns of that row a thread
-// stages; C = 32 / J tokens a chunk.
-template <typename T, int DQ, int J>
-__global__ __launch_bounds__(1024) void gla_scan_kernel(
+// rows are walked in chunks of C: all threads together bring a chunk's q, k, decay logits and v
+// from memory into registers, then into LDS as floats, the decay a = exp(log sigmoid(z) / tau)
+// computed on the way once an element; then every lane reads what it needs from LDS, a token at
+// a time, while the next chunk's loads are in flight.  Every load is issued unconditionally
+// (addresses clamped, values cleared when they are stored): a load whose result meets a constant
+// at the end of a branch would be waited for on the spot, one after the other.
+// LDS row of a token: q [KP] | k [KP] | a [KP] | v [VP], KP = 4 DQ >= key_dim and VP = 16 WAVES
+// >= value_dim, the padding zero (a padded key channel then adds nothing).
+template <int N> struct Pow2Up { static constexpr int value = N <= 16 ? 16 : N <= 32 ? 32 : N <= 64 ? 64 : N <= 128 ? 128 : 256; };
+
+template <typename T, int DQ, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gla_scan_kernel(
     float* __restrict__ o, const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k, int64_t k_stride,
     const T* __restrict__ v, int64_t v_stride, const float* __restrict__ z, float* __restrict__ state,
     const int* __restrict__ item_len, const int* __restrict__ item_tok_off, const int* __restrict__ item_slot,
     int heads, int key_dim, int value_dim, float scale, float inv_tau) {
-    constexpr int C = 32 / J, KP = 4 * DQ;
+    constexpr int KP = 4 * DQ, VP = 16 * WAVES, THREADS = 64 * WAVES, PER = 3 * KP + VP;
+    constexpr int C = PER > 512 ? 16 : 32;                       // rows a chunk: at most 64 KB of LDS
+    constexpr int KC = Pow2Up<KP>::value;                        // columns the threads are dealt over
+    constexpr int SK = (C * KC + THREADS - 1) / THREADS;         // loads a thread and chunk, per key array
+    constexpr int SV = (C * VP + THREADS - 1) / THREADS;         // and of v
     extern __shared__ float lds[];
     const int h = blockIdx.x, item = blockIdx.y;
     const int slot = item_slot[item], n = item_len[item];
     if (slot < 0 || n <= 0) return;                    // a padding item of a batch of fixed size
-    const int tid = threadIdx.x, threads = blockDim.x;
+    const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6, c16 = lane & 15, g = lane >> 4;
-    const int VP = threads >> 2, per = 3 * KP + VP;
     const int col = wave * 16 + c16;
     const bool col_ok = col < value_dim;
     const int d0 = g * DQ;
@@ -57,41 +63,58 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(
 #pragma unroll
     for (int i = 0; i < DQ; ++i) S[i] = (col_ok && d0 + i < key_dim) ? s_ptr[(int64_t)i * value_dim] : 0.f;
 
-    // the columns of the LDS row this thread stages: where each comes from (kind 0 q, 1 k, 2 z, 3 v, -1 padding)
-    int kind[J];
-    int64_t src[J], stride[J];
-#pragma unroll
-    for (int j = 0; j < J; ++j) {
-        const int e = tid + j * threads;
-        kind[j] = -1; src[j] = 0; stride[j] = 0;
-        if (e < 3 * KP) {
-            const int seg = e / KP, d = e - seg * KP;
-            if (d < key_dim) {
-                kind[j] = seg;
-                stride[j] = seg == 0 ? q_stride : seg == 1 ? k_stride : (int64_t)heads * key_dim;
-                src[j] = (int64_t)row0 * stride[j] + (int64_t)h * key_dim + d;
-            }
-        } else if (e < per && e - 3 * KP < value_dim) {
-            kind[j] = 3; stride[j] = v_stride;
-            src[j] = (int64_t)row0 * v_stride + (int64_t)h * value_dim + (e - 3 * KP);
-        }
-    }
-    float stage[J][C];
+    const T* qh = q + (int64_t)row0 * q_stride + (int64_t)h * key_dim;
+    const T* kh = k + (int64_t)row0 * k_stride + (int64_t)h * key_dim;
+    const T* vh = v + (int64_t)row0 * v_stride + (int64_t)h * value_dim;
+    const int64_t z_stride = (int64_t)heads * key_dim;
+    const float* zh = z + (int64_t)row0 * z_stride + (int64_t)h * key_dim;
+
+    T sq[SK], sk[SK], sv[SV];
+    float sz[SK];
     auto fetch = [&](int r0) {
+        const int left = n - r0;                       // rows of this chunk onwards (uniform)
 #pragma unroll
-        for (int j = 0; j < J; ++j)
-#pragma unroll
-            for (int r = 0; r < C; ++r) {
-                float x = 0.f;
-                if (r0 + r < n) {
-                    const int64_t at = src[j] + (int64_t)(r0 + r) * stride[j];
-                    if (kind[j] == 0) x = Elem<T>::load(q + at);
-                    else if (kind[j] == 1) x = Elem<T>::load(k + at);
-                    else if (kind[j] == 2) x = z[at];
-                    else if (kind[j] == 3) x = Elem<T>::load(v + at);
-                }
-                stage[j][r] = x;
+        for (int s = 0; s < SK; ++s) {
+            if ((s * THREADS) / KC < left) {           // else: a slot wholly behind the item's last row (uniform)
+                const int idx = tid + s * THREADS;
+                const int r = min(r0 + idx / KC, n - 1), d = min(idx % KC, key_dim - 1);
+                sq[s] = qh[(int64_t)r * q_stride + d];
+                sk[s] = kh[(int64_t)r * k_stride + d];
+                sz[s] = zh[(int64_t)r * z_stride + d];
             }
+        }
+#pragma unroll
+        for (int s = 0; s < SV; ++s) {
+            if ((s * THREADS) / VP < left) {
+                const int idx = tid + s * THREADS;
+                const int r = min(r0 + idx / VP, n - 1), d = min(idx % VP, value_dim - 1);
+                sv[s] = vh[(int64_t)r * v_stride + d];
+            }
+        }
+    };
+    auto put = [&](int r0) {
+        const int left = n - r0;
+#pragma unroll
+        for (int s = 0; s < SK; ++s) {
+            const int idx = tid + s * THREADS;
+            const int r = idx / KC, d = idx % KC;
+            if ((s * THREADS) / KC < left && r < C && d < KP) {
+                const bool ok = d < key_dim && r < left;
+                float* dst = lds + r * PER + d;
+                const float zz = sz[s];
+                // a = sigmoid(z)^(1/tau);  log sigmoid(z) = min(z, 0) - log(1 + exp(-|z|))
+                const float a = expf((fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)))) * inv_tau);
+                dst[0] = ok ? Elem<T>::load(&sq[s]) : 0.f;
+                dst[KP] = ok ? Elem<T>::load(&sk[s]) : 0.f;
+                dst[2 * KP] = ok ? a : 0.f;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < SV; ++s) {
+            const int idx = tid + s * THREADS;
+            const int r = idx / VP, d = idx % VP;
+            if ((s * THREADS) / VP < left && r < C) lds[r * PER + 3 * KP + d] = (d < value_dim && r < left) ? Elem<T>::load(&sv[s]) : 0.f;
+        }
     };
     float* op = o + ((int64_t)row0 * heads + h) * value_dim + col;
     const int64_t o_stride = (int64_t)heads * value_dim;
@@ -101,39 +124,40 @@ __global__ __launch_bounds__(1024) void gla_scan_kernel(
     fetch(0);
     for (int r0 = 0; r0 < n; r0 += C) {
         __syncthreads();                               // the chunk before has been read
-#pragma unroll
-        for (int j = 0; j < J; ++j) {
-            const int e = tid + j * threads;
-            if (e >= per) continue;
-#pragma unroll
-            for (int r = 0; r < C; ++r) {
-                float x = stage[j][r];
-                if (kind[j] == 2) {
-                    // a = sigmoid(z)^(1/tau);  log sigmoid(z) = min(z, 0) - log(1 + exp(-|z|))
-                    x = expf((fminf(x, 0.f) - log1pf(expf(-fabsf(x)))) * inv_tau);
-                }
-                lds[r * per + e] = x;
-            }
-        }
+        put(r0);
         __syncthreads();
         if (r0 + C < n) fetch(r0 + C);
         const int rows = min(C, n - r0);
+        // a row's operands are read from LDS while the row before it is computed
+        float4 q4[DQ / 4], k4[DQ / 4], a4[DQ / 4], qn[DQ / 4], kn[DQ / 4], an[DQ / 4];
+        float vv, vn;
+        auto read = [&](int r, float4* qq, float4* kk, float4* aa, float& v1) {
+            const float* row = lq + r * PER;
+#pragma unroll
+            for (int i = 0; i < DQ / 4; ++i) {
+                qq[i] = *reinterpret_cast<const float4*>(row + 4 * i);
+                kk[i] = *reinterpret_cast<const float4*>(row + KP + 4 * i);
+                aa[i] = *reinterpret_cast<const float4*>(row + 2 * KP + 4 * i);
+            }
+            v1 = lv[r * PER];
+        };
+        read(0, q4, k4, a4, vv);
         for (int r = 0; r < rows; ++r) {
-            const float* row = lq + r * per;
-            const float vv = lv[r * per];
+            read(min(r + 1, C - 1), qn, kn, an, vn);
             float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < DQ; i += 4) {
-                const float4 q4 = *reinterpret_cast<const float4*>(row + i);
-                const float4 k4 = *reinterpret_cast<const float4*>(row + KP + i);
-                const float4 a4 = *reinterpret_cast<const float4*>(row + 2 * KP + i);
-                S[i] = fmaf(a4.x, S[i], k4.x * vv);         acc = fmaf(S[i], q4.x, acc);
-                S[i + 1] = fmaf(a4.y, S[i + 1], k4.y * vv); acc = fmaf(S[i + 1], q4.y, acc);
-                S[i + 2] = fmaf(a4.z, S[i + 2], k4.z * vv); acc = fmaf(S[i + 2], q4.z, acc);
-                S[i + 3] = fmaf(a4.w, S[i + 3], k4.w * vv); acc = fmaf(S[i + 3], q4.w, acc);
+            for (int i = 0; i < DQ / 4; ++i) {
+                const int j = 4 * i;
+                S[j] = fmaf(a4[i].x, S[j], k4[i].x * vv);         acc = fmaf(S[j], q4[i].x, acc);
+                S[j + 1] = fmaf(a4[i].y, S[j + 1], k4[i].y * vv); acc = fmaf(S[j + 1], q4[i].y, acc);
+                S[j + 2] = fmaf(a4[i].z, S[j + 2], k4[i].z * vv); acc = fmaf(S[j + 2], q4[i].z, acc);
+                S[j + 3] = fmaf(a4[i].w, S[j + 3], k4[i].w * vv); acc = fmaf(S[j + 3], q4[i].w, acc);
             }
             acc = rows4_sum(acc);
             if (g == 0 && col_ok) op[(int64_t)(r0 + r) * o_stride] = acc * scale;
+#pragma unroll
+            for (int i = 0; i < DQ / 4; ++i) { q4[i] = qn[i]; k4[i] = kn[i]; a4[i] = an[i]; }
+            vv = vn;
         }
     }
 #pragma unroll
@@ -171,28 +195,27 @@ static int launch_gla_dq(float* o, const void* q, int64_t qs, const void* k, int
                          const float* z, float* state, const int* item_len, const int* item_tok_off,
                          const int* item_slot, int num_items, int heads, int key_dim, int value_dim, float scale,
                          float inv_tau, hipStream_t stream) {
-    const int waves = (value_dim + 15) / 16, threads = 64 * waves;
-    const int per = 3 * 4 * DQ + 16 * waves;
-    const int j = (per + threads - 1) / threads;
+    const int waves = (value_dim + 15) / 16;
     const dim3 grid(heads, num_items);
-    // (a chunk of the widest heads takes 128 KB of LDS, more than a launch gets without asking)
-#define ST_GLA(J)                                                                                                    \
+    // (a chunk takes up to 64 KB of LDS, more than a launch gets without asking)
+#define ST_GLA(W)                                                                                                    \
     {                                                                                                                \
-        const size_t bytes = (size_t)(32 / J) * per * sizeof(float);                                                 \
+        constexpr int per = 12 * DQ + 16 * W;                                                                        \
+        constexpr size_t bytes = (size_t)(per > 512 ? 16 : 32) * per * sizeof(float);                                \
         static bool asked = false;                                                                                   \
-        if (bytes > 48 * 1024 && !asked) {                                                                           \
-            ST_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gla_scan_kernel<T, DQ, J>),                  \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess,      \
+        if (bytes > 32 * 1024 && !asked) {                                                                           \
+            ST_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gla_scan_kernel<T, DQ, W>),                  \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) == hipSuccess,      \
                      "gla_scan: the device refuses %zu bytes of LDS", bytes);                                        \
             asked = true;                                                                                            \
         }                                                                                                            \
-        gla_scan_kernel<T, DQ, J><<<grid, threads, bytes, stream>>>(o, (const T*)q, qs, (const T*)k, ks,             \
+        gla_scan_kernel<T, DQ, W><<<grid, 64 * W, bytes, stream>>>(o, (const T*)q, qs, (const T*)k, ks,              \
             (const T*)v, vs, z, state, item_len, item_tok_off, item_slot, heads, key_dim, value_dim, scale, inv_tau);\
     }
-    if (j <= 1) ST_GLA(1)
-    else if (j <= 2) ST_GLA(2)
-    else if (j <= 4) ST_GLA(4)
-    else if (j <= 8) ST_GLA(8)
+    if (waves <= 1) ST_GLA(1)
+    else if (waves <= 2) ST_GLA(2)
+    else if (waves <= 4) ST_GLA(4)
+    else if (waves <= 8) ST_GLA(8)
     else ST_GLA(16)
 #undef ST_GLA
     ST_LAUNCH_CHECK("gla_scan");
@@ -213,7 +236,6 @@ static int launch_gla(float* o, const void* q, int64_t qs, const void* k, int64_
     if (dq <= 16) return launch_gla_dq<T, 16>(ST_GLA_ARGS);
     if (dq <= 24) return launch_gla_dq<T, 24>(ST_GLA_ARGS);
     if (dq <= 32) return launch_gla_dq<T, 32>(ST_GLA_ARGS);
-    if (dq <= 48) return launch_gla_dq<T, 48>(ST_GLA_ARGS);
     return launch_gla_dq<T, 64>(ST_GLA_ARGS);
 #undef ST_GLA_ARGS
 }

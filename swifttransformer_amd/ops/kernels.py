@@ -850,9 +850,11 @@ def latent_write(cache: torch.Tensor, x: torch.Tensor, gain: torch.Tensor, eps: 
 
 # ---------------------------------------------------------------- routed experts
 def moe_tile(num_tokens: int, top: int, experts: int) -> int:
-    """Places a tile: 64 where an expert gets some dozens of rows on average (a tile's weight
-    operands then meet four blocks of 16 rows), else 16 (few rows: only the weights' stream counts)."""
-    return 64 if num_tokens * top >= 32 * experts else 16
+    """Places a tile: 16 for few rows an expert (only the weights' stream counts), 64 or 128 where an
+    expert gets some dozens or a hundred rows on average (a tile's weight operands then meet four or
+    eight blocks of 16 rows, and the expert's weights are read once a tile)."""
+    pairs = num_tokens * top
+    return 128 if pairs >= 96 * experts else 64 if pairs >= 32 * experts else 16
 
 
 def moe_capacity(num_tokens: int, top: int, experts: int, tile: int) -> int:

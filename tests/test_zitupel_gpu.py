@@ -172,7 +172,7 @@ def test_gated_head_norm_and_latent_write(dtype):
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("T,W,F,E,top", [(37, 64, 48, 5, 2), (5, 72, 20, 7, 1), (64, 128, 64, 3, 3), (1, 40, 9, 4, 1),
-                                         (130, 33, 17, 6, 4)])
+                                         (130, 33, 17, 6, 4), (300, 64, 32, 3, 1)])
 def test_routed_experts(dtype, T, W, F, E, top):
     from swifttransformer_amd.ops import kernels as K
     dt = DTYPES[dtype]
