@@ -110,21 +110,25 @@ int st_token_conv_state(float* state, const float* x, const int* item_len, const
                         const int* item_slot, int num_items, int channels, int taps, hipStream_t stream);
 
 // ---- gated linear attention (csrc/recurrent.hip)
-// a = sigmoid(z)^(inv_tau), in place over n floats.
-int st_decay_gate(float* z, int64_t n, float inv_tau, hipStream_t stream);
+// out = sigmoid(z)^(inv_tau) over n floats (out may be z).
+int st_decay_gate(float* out, const float* z, int64_t n, float inv_tau, hipStream_t stream);
 // Per item and head, from the state S [key_dim, value_dim] of the item's slot and over its rows in
-// order: S = diag(a_t) S + k_t v_t^T with a_t = sigmoid(z_t)^(inv_tau), o_t = scale * S^T q_t; the
-// state is stored back.  q, k, v: rows of `dtype` with their strides in elements (head h at
-// h * key_dim / h * value_dim); z: float [T, heads * key_dim]; o: float [T, heads * value_dim];
-// state: float [slots, heads, key_dim, value_dim].
-int st_gla_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
-                const void* v, int64_t v_stride, const float* z, float* state,
-                const int* item_len, const int* item_tok_off, const int* item_slot, int num_items,
-                int heads, int key_dim, int value_dim, float scale, float inv_tau, int dtype, hipStream_t stream);
+// order: S = diag(a_t) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.  The key
+// channels are dealt to parts of part_dim (4, 8 or 16); part p writes its share of every o_t to
+// plane p of o_part [parts, T, heads * value_dim] (planes part_stride floats apart), and the sum
+// of the planes is o.  q, k, v: rows of `dtype` with their strides in elements (head h at
+// h * key_dim / h * value_dim); a: float [T, heads * key_dim]; state: float [slots, heads, key_dim, value_dim].
+int st_gla_scan(float* o_part, int64_t part_stride, int part_dim, const void* q, int64_t q_stride,
+                const void* k, int64_t k_stride, const void* v, int64_t v_stride, const float* a,
+                float* state, const int* item_len, const int* item_tok_off, const int* item_slot,
+                int num_items, int heads, int key_dim, int value_dim, float scale, int dtype, hipStream_t stream);
+int st_gla_scan_parts(int key_dim, int part_dim);
+// With o the sum of `parts` planes (part_stride floats apart):
 // out[t, h, j] = o[t, h, j] * rsqrt(mean_j o[t, h, :]^2 + eps) * gain[j] * silu(g[t, h, j]); g: rows
-// of `dtype` with stride g_stride; out: rows of `dtype`, dense.
-int st_gated_head_norm(void* out, const float* o, const void* g, int64_t g_stride, const float* gain,
-                       int num_tokens, int heads, int value_dim, float eps, int dtype, hipStream_t stream);
+// of `dtype` with stride g_stride; out: rows of `dtype`, dense.  Up to 256 value channels a head.
+int st_gated_head_norm(void* out, const float* o, int parts, int64_t part_stride, const void* g, int64_t g_stride,
+                       const float* gain, int num_tokens, int heads, int value_dim, float eps, int dtype,
+                       hipStream_t stream);
 
 // ---- latent cache (csrc/latent.hip)
 // Row t of x (float, stride x_stride, `rank` values) is normalised, c = x * rsqrt(mean x^2 + eps) *

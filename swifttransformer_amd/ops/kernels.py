@@ -68,10 +68,11 @@ def _lib():
         lib.st_token_conv.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int,
                                       _c_int, _c_p]
         lib.st_token_conv_state.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
-        lib.st_decay_gate.argtypes = [_c_p, _c_i64, _c_f, _c_p]
-        lib.st_gla_scan.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p,
-                                    _c_int, _c_int, _c_int, _c_int, _c_f, _c_f, _c_int, _c_p]
-        lib.st_gated_head_norm.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_decay_gate.argtypes = [_c_p, _c_p, _c_i64, _c_f, _c_p]
+        lib.st_gla_scan.argtypes = [_c_p, _c_i64, _c_int, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p,
+                                    _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_gated_head_norm.argtypes = [_c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int,
+                                           _c_f, _c_int, _c_p]
         lib.st_latent_write.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int,
                                         _c_int, _c_int, _c_f, _c_int, _c_p]
         lib.st_moe_route.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
@@ -757,34 +758,49 @@ def token_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx_a
 
 
 # ------------------------------------------------------ gated linear attention
-@_timed("decay_gate", lambda z, inv_tau: {"rows": z.shape[0], "width": z.shape[-1], "bytes": 8 * z.numel()})
-def decay_gate(z: torch.Tensor, inv_tau: float) -> torch.Tensor:
-    """In place: z <- sigmoid(z) ** inv_tau (float), computed as exp(inv_tau * log sigmoid(z))."""
+@_timed("decay_gate", lambda z, inv_tau, out=None: {"rows": z.shape[0], "width": z.shape[-1], "bytes": 8 * z.numel()})
+def decay_gate(z: torch.Tensor, inv_tau: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """sigmoid(z) ** inv_tau (float), computed as exp(inv_tau * log sigmoid(z)); in place unless ``out``."""
     _need(z, "z", torch.float32)
-    _check(_lib().st_decay_gate(_ptr(z), z.numel(), float(inv_tau), _stream()))
-    return z
+    if out is None:
+        out = z
+    _need(out, "out", torch.float32, z.shape)
+    _check(_lib().st_decay_gate(_ptr(out), _ptr(z), z.numel(), float(inv_tau), _stream()))
+    return out
 
 
-def _d_gla_scan(q, k, v, gate, state, ctx_arrays, heads, scale, inv_tau):
+class PartialSums:
+    """A result still split into planes that are to be summed: ``planes`` float [parts, T, width]."""
+
+    def __init__(self, planes: torch.Tensor):
+        self.planes = planes
+
+    def sum(self) -> torch.Tensor:
+        return self.planes.sum(0)
+
+
+def _d_gla_scan(q, k, v, decay, state, ctx_arrays, heads, scale, part_dim=0):
     T = q.shape[0]
     kd, vd = q.shape[1] // heads, v.shape[1] // heads
-    return {"rows": T, "heads": heads, "key_dim": kd, "value_dim": vd, "items": ctx_arrays[2].shape[0],
+    parts = -(-kd // (part_dim or 16))
+    return {"rows": T, "heads": heads, "key_dim": kd, "value_dim": vd, "items": ctx_arrays[2].shape[0], "parts": parts,
             "flops": 4 * T * heads * kd * vd,
-            # operands and results of every row, and the items' states read and written once
-            "bytes": T * heads * ((2 * kd + vd) * q.element_size() + 4 * kd + 4 * vd) +
+            # operands of every row, the planes of partial results, and the items' states read and written once
+            "bytes": T * heads * ((2 * kd + vd) * q.element_size() + 4 * kd + 4 * vd * parts) +
                      8 * ctx_arrays[2].shape[0] * heads * kd * vd}
 
 
 @_timed("gla_scan", _d_gla_scan)
-def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor, state: torch.Tensor,
-             ctx_arrays, heads: int, scale: float, inv_tau: float) -> torch.Tensor:
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
+             ctx_arrays, heads: int, scale: float, part_dim: int = 0) -> PartialSums:
     """Per item and head, from the slot's state S and over the item's rows in order:
-    S <- diag(a_t) S + k_t v_t^T with the decay a_t = sigmoid(gate_t) ** inv_tau, o_t = scale * S^T q_t;
-    the state is stored back.
+    S <- diag(decay_t) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.
 
     q, k: [T, heads * key_dim], v: [T, heads * value_dim] views (dense rows, any row stride);
-    gate: float [T, heads * key_dim]; state: float [slots, heads, key_dim, value_dim].  Returns
-    float [T, heads * value_dim]."""
+    decay: float [T, heads * key_dim]; state: float [slots, heads, key_dim, value_dim].  The key
+    channels are dealt to parts of ``part_dim`` (4, 8 or 16; 0: 16); the result
+    comes as the parts' planes [parts, T, heads * value_dim], whose sum is o (``gated_head_norm``
+    sums them)."""
     _token_item, item_len, item_tok_off, item_slot = ctx_arrays
     T = q.shape[0]
     kd, vd = q.shape[1] // heads, v.shape[1] // heads
@@ -792,34 +808,39 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tens
         _need(t, name, q.dtype, (T, w), contiguous=False)
         if t.stride(1) != 1:
             raise KernelError(f"{name}: rows must be dense")
-    _need(gate, "gate", torch.float32, (T, heads * kd))
+    _need(decay, "decay", torch.float32, (T, heads * kd))
     _need(state, "state", torch.float32, (state.shape[0], heads, kd, vd))
     B = item_slot.shape[0]
     for name, t in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
         _need(t, name, torch.int32, (B,))
-    out = empty((T, heads * vd), torch.float32, q.device)
-    _check(_lib().st_gla_scan(_ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
-                              _ptr(gate), _ptr(state), _ptr(item_len), _ptr(item_tok_off), _ptr(item_slot), B,
-                              heads, kd, vd, float(scale), float(inv_tau), dtype_code(q.dtype), _stream()))
-    return out
+    part_dim = int(part_dim) or 16
+    parts = -(-kd // part_dim)
+    planes = empty((parts, T, heads * vd), torch.float32, q.device)
+    _check(_lib().st_gla_scan(_ptr(planes), T * heads * vd, part_dim, _ptr(q), q.stride(0), _ptr(k), k.stride(0),
+                              _ptr(v), v.stride(0), _ptr(decay), _ptr(state), _ptr(item_len), _ptr(item_tok_off),
+                              _ptr(item_slot), B, heads, kd, vd, float(scale), dtype_code(q.dtype), _stream()))
+    return PartialSums(planes)
 
 
-@_timed("gated_head_norm", lambda o, gate, *a, **k: {"rows": o.shape[0], "width": o.shape[1],
-                                                     "bytes": o.numel() * (4 + 2 * gate.element_size())})
-def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, heads: int, eps: float,
+@_timed("gated_head_norm", lambda o, gate, *a, **k: {
+    "rows": gate.shape[0], "width": gate.shape[1],
+    "bytes": gate.numel() * (2 * gate.element_size() + 4 * (o.planes.shape[0] if isinstance(o, PartialSums) else 1))})
+def gated_head_norm(o, gate: torch.Tensor, gain: torch.Tensor, heads: int, eps: float,
                     out_dtype: torch.dtype) -> torch.Tensor:
     """out[t, h, :] = o[t, h, :] * rsqrt(mean(o[t, h, :]^2) + eps) * gain * silu(gate[t, h, :]).
-    o: float [T, heads * value_dim]; gate: a view of ``out_dtype`` rows; gain: float [value_dim]."""
-    T = o.shape[0]
-    vd = o.shape[1] // heads
-    _need(o, "o", torch.float32, (T, heads * vd))
+    o: float [T, heads * value_dim], or the ``PartialSums`` whose planes sum to it; gate: a view of
+    ``out_dtype`` rows; gain: float [value_dim]."""
+    planes = o.planes if isinstance(o, PartialSums) else o.unsqueeze(0)
+    parts, T, width = planes.shape
+    vd = width // heads
+    _need(planes, "o", torch.float32, (parts, T, heads * vd))
     _need(gate, "gate", out_dtype, (T, heads * vd), contiguous=False)
     if gate.stride(1) != 1:
         raise KernelError("gate: rows must be dense")
     _need(gain, "gain", torch.float32, (vd,))
-    out = empty((T, heads * vd), out_dtype, o.device)
-    _check(_lib().st_gated_head_norm(_ptr(out), _ptr(o), _ptr(gate), gate.stride(0), _ptr(gain), T, heads, vd,
-                                     float(eps), dtype_code(out_dtype), _stream()))
+    out = empty((T, heads * vd), out_dtype, planes.device)
+    _check(_lib().st_gated_head_norm(_ptr(out), _ptr(planes), parts, T * width, _ptr(gate), gate.stride(0),
+                                     _ptr(gain), T, heads, vd, float(eps), dtype_code(out_dtype), _stream()))
     return out
 
 

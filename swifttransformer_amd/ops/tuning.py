@@ -38,6 +38,13 @@ class Tuning:
     # (FC2 at 512 rows 202 -> 156 us, FC1 at 2,048 rows 465 -> 365 us: a layer 8 to 10 % faster),
     # so every recording times them.
     tune_products_up_to_rows: int = 1 << 20
+    # Key channels a wave of the gated-linear-attention scan takes (4, 8 or 16): in steps of single
+    # tokens, where the requests are many and the states' traffic counts, and in steps with prompt
+    # portions, where a portion's tokens come one after the other and more parts a head are more
+    # compute units at work on them (every part writes a plane of partial results, which the head
+    # norm sums).
+    gla_part_dim_decode: int = 16
+    gla_part_dim_prompt: int = 8
 
 
 tuning = Tuning()

@@ -114,31 +114,37 @@ def test_gla_scan_whole_portions_and_single_tokens(dtype, heads, kd, vd):
     q, k, v = rnd(T, heads, kd), rnd(T, heads, kd) * 0.5, rnd(T, heads, vd)
     z = torch.randn(T, heads * kd, generator=g) * 2 + 1
     a = torch.sigmoid(z.to(F64)).pow(1 / 3.0)
-    check(K.decay_gate(dev(z), 1 / 3.0), a.numpy(), torch.float32, "decay gate")
-    decay = dev(z)                                                       # the scan takes the logits
+    decay = K.decay_gate(dev(z), 1 / 3.0)
+    check(decay, a.numpy(), torch.float32, "decay gate")
     want, S_end = plain_scan(q, k, v, a.view(T, heads, kd), torch.zeros(heads, kd, vd, dtype=F64), 0.37)
     # one fused row [q | junk | k | v] so that the operands are strided views
     fused = torch.cat([q.reshape(T, -1), torch.full((T, 8), float("nan"), dtype=F64), k.reshape(T, -1), v.reshape(T, -1)], 1)
     fused = dev(fused, dt)
     o0, o1, o2 = heads * kd, heads * kd + 8, 2 * heads * kd + 8
-    for cuts in ([T], [1] * T, [2, 5, 1, 15]):
+    odt = torch.float32 if dt == torch.float32 else dt
+    for cuts, part_dim in (([T], 0), ([1] * T, 0), ([2, 5, 1, 15], 4), ([T], 16), ([7, 16], 8)):
         state = torch.zeros((2, heads, kd, vd), device=DEV)
         state[0] = float("nan")                                          # another request's slot is not touched
         got, lo = [], 0
         for n in cuts:
             rows = fused[lo:lo + n]
             got.append(K.gla_scan(rows[:, :o0], rows[:, o1:o2], rows[:, o2:], decay[lo:lo + n], state,
-                                  items_ctx([n], [1]), heads, 0.37, 1 / 3.0))
+                                  items_ctx([n], [1]), heads, 0.37, part_dim).sum())
             lo += n
-        what = f"{dtype} heads {heads} key {kd} value {vd} cuts {cuts[:4]}"
-        check(torch.cat(got), want.reshape(T, -1).numpy(), torch.float32 if dt == torch.float32 else dt, what)
+        what = f"{dtype} heads {heads} key {kd} value {vd} cuts {cuts[:4]} parts of {part_dim}"
+        check(torch.cat(got), want.reshape(T, -1).numpy(), odt, what)
         check(state[1], S_end.numpy(), torch.float32, what + " state")
         assert torch.isnan(state[0]).all()
-    # two items in one launch, the second a padding item
+    # two items in one launch, the second a padding item; the planes summed by the head norm's kernel
     state = torch.zeros((2, heads, kd, vd), device=DEV)
     ti, ln, off, sl = items_ctx([T, 0], [0, -1])
-    got = K.gla_scan(fused[:, :o0], fused[:, o1:o2], fused[:, o2:], decay, state, (ti, ln, off, sl), heads, 0.37, 1 / 3.0)
-    check(got, want.reshape(T, -1).numpy(), torch.float32 if dt == torch.float32 else dt, "with a padding item")
+    planes = K.gla_scan(fused[:, :o0], fused[:, o1:o2], fused[:, o2:], decay, state, (ti, ln, off, sl), heads, 0.37)
+    check(planes.sum(), want.reshape(T, -1).numpy(), odt, "with a padding item")
+    gate = torch.randn(T, heads * vd).to(dt)
+    gain = torch.rand(vd) + 0.5
+    gg = gate.to(F64)
+    normed = (plain.unit(want, 1e-4) * gain.to(F64)).reshape(T, -1) * (gg / (1 + torch.exp(-gg)))
+    check(K.gated_head_norm(planes, dev(gate, dt), dev(gain), heads, 1e-4, dt), normed.numpy(), dt, "head norm of the planes")
 
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
