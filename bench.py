@@ -575,7 +575,7 @@ def main() -> int:
     ap.add_argument("--workload", default="decode-1.3b",
                     choices=["decode-1.3b", "mixed-6.7b", "mixed-1.3b", "ttft", "decode-30b", "decode-family",
                              "zitupel-125m", "zitupel-1.3b", "zitupel-6.7b"],
-                    help="decode-1.3b is the contract's line; the others are the other model shapes; zitupel-<size>: "
+                    help="decode-1.3b is the default line; the others are the other model shapes; zitupel-<size>: "
                          "the Zitupel architecture beside OPT at the same layer sizes")
     args = ap.parse_args()
     if args.gpus != 1:
