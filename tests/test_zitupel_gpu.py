@@ -109,7 +109,7 @@ def test_gla_scan_whole_portions_and_single_tokens(dtype, heads, kd, vd):
     from swifttransformer_amd.ops import kernels as K
     dt = DTYPES[dtype]
     g = torch.Generator().manual_seed(kd + vd)
-    T = 23
+    T = 70                                                              # the scan walks in chunks of 32 tokens
     rnd = lambda *s: torch.randn(*s, generator=g).to(dt).to(F64)        # values the storage type holds
     q, k, v = rnd(T, heads, kd), rnd(T, heads, kd) * 0.5, rnd(T, heads, vd)
     z = torch.randn(T, heads * kd, generator=g) * 2 + 1
@@ -122,7 +122,9 @@ def test_gla_scan_whole_portions_and_single_tokens(dtype, heads, kd, vd):
     fused = dev(fused, dt)
     o0, o1, o2 = heads * kd, heads * kd + 8, 2 * heads * kd + 8
     odt = torch.float32 if dt == torch.float32 else dt
-    for cuts, part_dim in (([T], 0), ([1] * T, 0), ([2, 5, 1, 15], 4), ([T], 16), ([7, 16], 8)):
+    # (portions that end just before, at and just behind the edges of the scan's chunks)
+    for cuts, part_dim in (([T], 0), ([1] * T, 0), ([2, 5, 1, 23, 1, 32, 6], 4), ([T], 16), ([33, 31, 6], 8), ([64, 6], 8),
+                           ([65, 5], 16)):
         state = torch.zeros((2, heads, kd, vd), device=DEV)
         state[0] = float("nan")                                          # another request's slot is not touched
         got, lo = [], 0
@@ -203,6 +205,18 @@ def test_routed_experts(dtype, T, W, F, E, top):
                            out_scale=m, token_item=token_item)
     assert got.data_ptr() == r.data_ptr()
     check(got, want.numpy(), dt, f"{dtype} T {T} W {W} F {F} E {E} top {top}")
+    # every row to the same experts: one expert's tiles fill up and run over by one row
+    for rows in (t for t in (16, 17, 64, 65, 129) if t <= T):
+        same = torch.arange(E, dtype=torch.float32).flip(0).repeat(rows, 1) * 3
+        r1 = dev(res[:rows])
+        got = K.routed_experts(dev(x[:rows], dt), dev(same), dev(wg, dt), dev(wu, dt), dev(wd, dt), r1, top=top, limit=limit,
+                               out_scale=m)
+        s1 = torch.sigmoid(same[0].to(F64))
+        want1 = res[:rows].to(F64).clone()
+        for t in range(rows):
+            for e in range(top):
+                want1[t] += m * plain.expert(s1[e] * x[t], w, f"e{e}.", limit)
+        check(got, want1.numpy(), dt, f"{dtype} {rows} rows to the same {top} experts")
     # padding rows keep what they held
     r2 = dev(res)
     token_item[T // 2:] = -1
