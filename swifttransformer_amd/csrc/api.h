@@ -38,7 +38,7 @@ int st_activation_multiply(void* out, int64_t out_stride, const void* a, int64_t
 
 struct StGemmExtras;
 // activation: the function between bias and residual, by number (csrc/activation.h): 0 none,
-// 1 ReLU, 2 SiLU, 3 GELU in its tanh form, 4 GELU in its exact (erf) form, 5 log sigmoid; others are refused.
+// 1 ReLU, 2 SiLU, 3 GELU in its tanh form, 4 GELU in its exact (erf) form; others are refused.
 int st_gemm(void* out, const void* x, const void* w, const float* bias, const float* residual,
             int M, int N, int K, int activation, int dtype, int out_f32, int algo,
             const StGemmExtras* extras, hipStream_t stream);
@@ -110,15 +110,16 @@ int st_token_conv_state(float* state, const float* x, const int* item_len, const
                         const int* item_slot, int num_items, int channels, int taps, hipStream_t stream);
 
 // ---- gated linear attention (csrc/recurrent.hip)
+// out = sigmoid(z)^(inv_tau) over n floats (out may be z).
+int st_decay_gate(float* out, const float* z, int64_t n, float inv_tau, hipStream_t stream);
 // Per item and head, from the state S [key_dim, value_dim] of the item's slot and over its rows in
-// order: S = diag(a_t) S + k_t v_t^T with a_t = exp(log_a_t), o_t = scale * S^T q_t; the state is stored back.  The key
+// order: S = diag(a_t) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.  The key
 // channels are dealt to parts of part_dim (4, 8 or 16); part p writes its share of every o_t to
 // plane p of o_part [parts, T, heads * value_dim] (planes part_stride floats apart), and the sum
 // of the planes is o.  q, k, v: rows of `dtype` with their strides in elements (head h at
-// h * key_dim / h * value_dim); log_a: float [T, heads * key_dim], the decays' logarithms; state: float
-// [slots, heads, key_dim, value_dim].
+// h * key_dim / h * value_dim); a: float [T, heads * key_dim]; state: float [slots, heads, key_dim, value_dim].
 int st_gla_scan(float* o_part, int64_t part_stride, int part_dim, const void* q, int64_t q_stride,
-                const void* k, int64_t k_stride, const void* v, int64_t v_stride, const float* log_a,
+                const void* k, int64_t k_stride, const void* v, int64_t v_stride, const float* a,
                 float* state, const int* item_len, const int* item_tok_off, const int* item_slot,
                 int num_items, int heads, int key_dim, int value_dim, float scale, int dtype, hipStream_t stream);
 int st_gla_scan_parts(int key_dim, int part_dim);

@@ -1,7 +1,6 @@
 // Gated linear attention: a matrix-valued state per request and head that decays per key channel.
 //
 //   S_t = diag(a_t) S_(t-1) + k_t v_t^T          S: [key_dim, value_dim], float, one per (slot, head)
-//                                                 a_t = exp(log a_t); the logarithm is what comes in
 //   o_t = scale * S_t^T q_t
 //
 // One kernel serves whole prompts, portions and single decoded tokens: it loads the state of the
@@ -23,8 +22,16 @@
 
 namespace st {
 
+__global__ __launch_bounds__(256) void decay_gate_out_kernel(float* __restrict__ out, const float* __restrict__ z,
+                                                             int64_t n, float inv_tau) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = z[i];
+    out[i] = expf((fminf(v, 0.f) - log1pf(expf(-fabsf(v)))) * inv_tau);
+}
+
 // grid (heads * parts, ceil(value_dim / 64), items), one wave a workgroup.  LDS row of a token:
-// q [DQ] | k [DQ] | a [DQ] (a = exp of the logarithm that comes in) of this wave's part, the part's tail (key channels the head does not
+// q [DQ] | k [DQ] | a [DQ] of this wave's part, the part's tail (key channels the head does not
 // have) zero.  Loads are issued unconditionally, addresses clamped: a load whose result meets a
 // constant at the end of a branch would be waited for on the spot.
 template <typename T, int DQ>
@@ -88,7 +95,7 @@ __global__ __launch_bounds__(64) void gla_scan_kernel(
             float* dst = lds + r * (3 * DQ) + d;
             dst[0] = ok ? Elem<T>::load(&sq[s]) : 0.f;
             dst[DQ] = ok ? Elem<T>::load(&sk[s]) : 0.f;
-            dst[2 * DQ] = ok ? expf(sa[s]) : 0.f;      // the decay from its logarithm, once an element
+            dst[2 * DQ] = ok ? sa[s] : 0.f;
         }
         float vv[C];
 #pragma unroll
@@ -173,6 +180,15 @@ static int launch_gla(float* o_part, int64_t part_stride, const void* q, int64_t
 }  // namespace st
 
 using namespace st;
+
+extern "C" int st_decay_gate(float* out, const float* z, int64_t n, float inv_tau, hipStream_t stream) {
+    ST_CHECK(n >= 0 && ((z && out) || n == 0), "decay_gate: bad operands");
+    ST_CHECK(inv_tau > 0.f, "decay_gate: the exponent must be positive");
+    if (n == 0) return 0;
+    decay_gate_out_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(out, z, n, inv_tau);
+    ST_LAUNCH_CHECK("decay_gate");
+    return 0;
+}
 
 extern "C" int st_gla_scan_parts(int key_dim, int part_dim) {
     return part_dim > 0 ? (key_dim + part_dim - 1) / part_dim : 0;

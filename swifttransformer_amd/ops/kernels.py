@@ -68,6 +68,7 @@ def _lib():
         lib.st_token_conv.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int,
                                       _c_int, _c_p]
         lib.st_token_conv_state.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_decay_gate.argtypes = [_c_p, _c_p, _c_i64, _c_f, _c_p]
         lib.st_gla_scan.argtypes = [_c_p, _c_i64, _c_int, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p,
                                     _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
         lib.st_gated_head_norm.argtypes = [_c_p, _c_p, _c_int, _c_i64, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int,
@@ -340,8 +341,7 @@ def wide_offered(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
 
 # functions of the products' epilogues and of ``activation_multiply``, by the C interface's number
 # (csrc/activation.h; the names config files use for them)
-ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3, "gelu": 4, "gelu_erf": 4,
-               "log_sigmoid": 5}
+ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3, "gelu": 4, "gelu_erf": 4}
 
 
 def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_f32=False, algo=0,
@@ -758,6 +758,17 @@ def token_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx_a
 
 
 # ------------------------------------------------------ gated linear attention
+@_timed("decay_gate", lambda z, inv_tau, out=None: {"rows": z.shape[0], "width": z.shape[-1], "bytes": 8 * z.numel()})
+def decay_gate(z: torch.Tensor, inv_tau: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """sigmoid(z) ** inv_tau (float), computed as exp(inv_tau * log sigmoid(z)); in place unless ``out``."""
+    _need(z, "z", torch.float32)
+    if out is None:
+        out = z
+    _need(out, "out", torch.float32, z.shape)
+    _check(_lib().st_decay_gate(_ptr(out), _ptr(z), z.numel(), float(inv_tau), _stream()))
+    return out
+
+
 class PartialSums:
     """A result still split into planes that are to be summed: ``planes`` float [parts, T, width]."""
 
@@ -768,7 +779,7 @@ class PartialSums:
         return self.planes.sum(0)
 
 
-def _d_gla_scan(q, k, v, log_decay, state, ctx_arrays, heads, scale, part_dim=0):
+def _d_gla_scan(q, k, v, decay, state, ctx_arrays, heads, scale, part_dim=0):
     T = q.shape[0]
     kd, vd = q.shape[1] // heads, v.shape[1] // heads
     parts = -(-kd // (part_dim or 16))
@@ -780,13 +791,13 @@ def _d_gla_scan(q, k, v, log_decay, state, ctx_arrays, heads, scale, part_dim=0)
 
 
 @_timed("gla_scan", _d_gla_scan)
-def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_decay: torch.Tensor, state: torch.Tensor,
+def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
              ctx_arrays, heads: int, scale: float, part_dim: int = 0) -> PartialSums:
     """Per item and head, from the slot's state S and over the item's rows in order:
-    S <- diag(exp(log_decay_t)) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.
+    S <- diag(decay_t) S + k_t v_t^T, o_t = scale * S^T q_t; the state is stored back.
 
     q, k: [T, heads * key_dim], v: [T, heads * value_dim] views (dense rows, any row stride);
-    log_decay: float [T, heads * key_dim], the decays' logarithms (<= 0); state: float [slots, heads, key_dim, value_dim].  The key
+    decay: float [T, heads * key_dim]; state: float [slots, heads, key_dim, value_dim].  The key
     channels are dealt to parts of ``part_dim`` (4, 8 or 16; 0: 16); the result
     comes as the parts' planes [parts, T, heads * value_dim], whose sum is o (``gated_head_norm``
     sums them)."""
@@ -797,7 +808,7 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_decay: torch
         _need(t, name, q.dtype, (T, w), contiguous=False)
         if t.stride(1) != 1:
             raise KernelError(f"{name}: rows must be dense")
-    _need(log_decay, "log_decay", torch.float32, (T, heads * kd))
+    _need(decay, "decay", torch.float32, (T, heads * kd))
     _need(state, "state", torch.float32, (state.shape[0], heads, kd, vd))
     B = item_slot.shape[0]
     for name, t in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
@@ -806,7 +817,7 @@ def gla_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_decay: torch
     parts = -(-kd // part_dim)
     planes = empty((parts, T, heads * vd), torch.float32, q.device)
     _check(_lib().st_gla_scan(_ptr(planes), T * heads * vd, part_dim, _ptr(q), q.stride(0), _ptr(k), k.stride(0),
-                              _ptr(v), v.stride(0), _ptr(log_decay), _ptr(state), _ptr(item_len), _ptr(item_tok_off),
+                              _ptr(v), v.stride(0), _ptr(decay), _ptr(state), _ptr(item_len), _ptr(item_tok_off),
                               _ptr(item_slot), B, heads, kd, vd, float(scale), dtype_code(q.dtype), _stream()))
     return PartialSums(planes)
 

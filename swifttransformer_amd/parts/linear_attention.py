@@ -74,11 +74,9 @@ class GatedLinearAttention(Mixer):
         qk, vs = self.qk_size, self.v_size
         proj = K.gemm(x_t, self.w_in)
         low = K.gemm(x_t, self.w_decay_in)
-        # the decay's logarithm, log sigmoid(.) / tau, from the product's own epilogue in float
-        log_decay = K.gemm(low, self.w_decay_out, bias=self.b_decay, activation="log_sigmoid", out_f32=True,
-                           out_scale=1.0 / self.tau)
+        decay = K.decay_gate(K.gemm(low, self.w_decay_out, bias=self.b_decay, out_f32=True), 1.0 / self.tau)
         items = (ctx.token_item, ctx.item_len, ctx.item_tok_off, ctx.item_slot)
-        o = K.gla_scan(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + vs], log_decay, cache.state, items,
+        o = K.gla_scan(proj[:, :qk], proj[:, qk:2 * qk], proj[:, 2 * qk:2 * qk + vs], decay, cache.state, items,
                        self.num_heads, self.scale,
                        tuning.gla_part_dim_decode if ctx.all_single else tuning.gla_part_dim_prompt)
         y = K.gated_head_norm(o, proj[:, 2 * qk + vs:], self.gain, self.num_heads, self.eps, self.dtype)

@@ -114,7 +114,8 @@ def test_gla_scan_whole_portions_and_single_tokens(dtype, heads, kd, vd):
     q, k, v = rnd(T, heads, kd), rnd(T, heads, kd) * 0.5, rnd(T, heads, vd)
     z = torch.randn(T, heads * kd, generator=g) * 2 + 1
     a = torch.sigmoid(z.to(F64)).pow(1 / 3.0)
-    decay = dev(torch.log(a))                                            # the scan takes the decays' logarithms
+    decay = K.decay_gate(dev(z), 1 / 3.0)
+    check(decay, a.numpy(), torch.float32, "decay gate")
     want, S_end = plain_scan(q, k, v, a.view(T, heads, kd), torch.zeros(heads, kd, vd, dtype=F64), 0.37)
     # one fused row [q | junk | k | v] so that the operands are strided views
     fused = torch.cat([q.reshape(T, -1), torch.full((T, 8), float("nan"), dtype=F64), k.reshape(T, -1), v.reshape(T, -1)], 1)
@@ -238,11 +239,6 @@ def test_scaled_residual_and_exact_gelu_in_the_products(dtype, M):
     check(got, (res.to(F64) + 0.3 * u).numpy(), dt, "scaled into the residual")
     got = K.gemm(dev(x, dt), dev(w, dt), activation="gelu")
     check(got, (0.5 * u * (1 + torch.erf(u / math.sqrt(2)))).numpy(), dt, "exact gelu")
-    # a decay's logarithm over a temperature: bias, log sigmoid and the factor in one epilogue, float result
-    bias = torch.randn(96, generator=g) * 3
-    got = K.gemm(dev(x, dt), dev(w, dt) * 8, bias=dev(bias), activation="log_sigmoid", out_f32=True, out_scale=0.25)
-    u8 = x.to(F64) @ (w.to(F64) * 8).T + bias.to(F64)
-    check(got, (0.25 * torch.nn.functional.logsigmoid(u8)).numpy(), dt, "log sigmoid over a temperature")
 
 
 # ------------------------------------------------------------- the engine on models
