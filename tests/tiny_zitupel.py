@@ -6,7 +6,9 @@ P: latent attention first (own latent, no feed-forward), gated linear attention 
    gated linear attention with tau 1 and all of three experts; three taps; factor 0.7.
 Q: sizes that no vector load divides (key size 10, value size 12, rank 40, width 72, inner widths
    50 and 20), one expert a token, five taps, two latent owners and two borrowers of the second.
-R: no convolution, factor 1, eight taps are not there to be had; a latent layer last; tau 64.
+R: no convolution, factor 1; a latent layer last; tau 64; wide heads (128 key channels).
+S: a width of 90 (no multiple of 4), two taps, head sizes 6 x 18 and 20 x 36, a rank of 20 in entries
+   of 32, a decay rank of 5, inner widths 30, 70 and 10.
 """
 from __future__ import annotations
 
@@ -55,9 +57,15 @@ CONFIGS = {
           "layers": [_with(_gla(4, 32, 32, 64.0), _moe(6, 2, 64, 4.0)),
                      _with(_gla(2, 128, 48, 2.0), None),
                      _with(_lat(2, 64, 64, 128, 0.6), {"kind": "dense", "ff": 40})]},
+    "S": {"architecture": "Zitupel", "vocab": 77, "width": 90, "residual_mult": 0.6, "norm": {"eps": 1e-5},
+          "canon": {"taps": 2},
+          "layers": [_with(_gla(2, 20, 36, 3.0), _moe(3, 1, 30, 2.0)),
+                     _with(_lat(3, 24, 40, 20, 0.3), {"kind": "dense", "ff": 70}),
+                     _with(_gla(5, 6, 18, 16.0), _moe(4, 2, 10, 1.2)),
+                     _with(_lat(1, 16, 16, 20, 0.5, src=1), None)]},
 }
-DECAY_RANK = {"P": 8, "Q": 6, "R": 16}
-PAGE_SIZE = {"P": 4, "Q": 2, "R": 16}
+DECAY_RANK = {"P": 8, "Q": 6, "R": 16, "S": 5}
+PAGE_SIZE = {"P": 4, "Q": 2, "R": 16, "S": 8}
 
 
 def make_weights(cfg: dict, seed: int, decay_rank: int, clean_routing: bool = False) -> Dict[str, torch.Tensor]:
