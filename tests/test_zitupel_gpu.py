@@ -104,7 +104,7 @@ def plain_scan(q, k, v, a, S, scale):
 
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
-@pytest.mark.parametrize("heads,kd,vd", [(3, 48, 32), (2, 10, 12), (1, 128, 80), (2, 256, 16), (4, 4, 100)])
+@pytest.mark.parametrize("heads,kd,vd", [(3, 56, 24), (2, 10, 12), (1, 128, 80), (2, 256, 16), (4, 4, 100)])
 def test_gla_scan_whole_portions_and_single_tokens(dtype, heads, kd, vd):
     from swifttransformer_amd.ops import kernels as K
     dt = DTYPES[dtype]
