@@ -32,7 +32,8 @@ class DeviceCache:
                 shape = (n, g.pool.num_pages, g.need.num_kv_heads, manager.page_size, g.need.head_dim)
                 k = torch.full(shape, fill, dtype=dtype, device=device)
                 if g.need.values:
-                    v = torch.full(shape, fill, dtype=dtype, device=device)
+                    vshape = shape[:-1] + (g.need.value_dim or g.need.head_dim,)
+                    v = torch.full(vshape, fill, dtype=dtype, device=device)
                     self.pools[g.index] = (k, v)
                 else:                       # one vector a token is key and value: the views' v is their k
                     v = k

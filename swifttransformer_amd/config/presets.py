@@ -73,3 +73,40 @@ def zitupel_preset(name: str, **overrides):
                         max_positions=2048)
     fields.update(overrides)
     return ZitupelHyperParam(**fields).validate()
+
+
+# ---- named sizes of the Zimorax family, for runs with random weights: the layer sizes of the OPT
+# model of the same name (width, heads, feed-forward width).  Of every four layers the first is a gated
+# delta rule, the second windowed attention (a quarter of the heads as key heads, a window of 1,024,
+# rotary positions on half of each head, scaled fourfold), the last two state-space mixers; the first
+# two layers run twice.
+def zimorax_preset(name: str, **overrides):
+    from .zimorax_param import ZimoraxHyperParam
+    key = name.lower().replace("-", "_")
+    size = key.split("_", 1)[1] if "_" in key else ""
+    if "opt_" + size not in _SIZES:
+        raise KeyError(f"invalid model name {name!r}; valid names: " +
+                       " ".join("zimorax_" + k.split("_", 1)[1] for k in _SIZES))
+    n_layers, hidden, heads, ffn = _SIZES["opt_" + size]
+    n_layers = int(overrides.pop("num_layers", n_layers))
+    only = overrides.pop("only", None)            # one mixer type for every layer (measurements)
+    window = int(overrides.pop("window", 1024))
+    loop_times = int(overrides.pop("loop_times", 2))
+    hd = hidden // heads
+    layers = []
+    for i in range(n_layers):
+        kind = only or ("delta", "attention", "mamba2", "mamba2")[i % 4]
+        if kind == "attention":
+            mixer = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": hd, "vdim": hd, "scale": float(hd) ** -0.5,
+                     "mask": {"size": window},
+                     "rot": {"dims": hd // 2, "base": 10000.0,
+                             "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+        elif kind == "mamba2":
+            mixer = {"heads": heads, "vdim": hd, "state": 64, "groups": max(1, heads // 8), "norm_groups": 1, "conv": 4}
+        else:
+            mixer = {"heads": heads, "kv_heads": heads, "dim": hd, "vdim": hd, "conv": 4}
+        layers.append({"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": ffn}})
+    loop = {"start": 0, "stop": min(2, n_layers), "times": loop_times} if loop_times > 0 else None
+    fields: Dict = dict(vocab=50272, width=hidden, layers=layers, loop=loop, norm_eps=1e-5, max_positions=4096)
+    fields.update(overrides)
+    return ZimoraxHyperParam(**fields).validate()

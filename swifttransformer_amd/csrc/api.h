@@ -38,7 +38,7 @@ int st_activation_multiply(void* out, int64_t out_stride, const void* a, int64_t
 
 struct StGemmExtras;
 // activation: the function between bias and residual, by number (csrc/activation.h): 0 none,
-// 1 ReLU, 2 SiLU, 3 GELU in its tanh form, 4 GELU in its exact (erf) form; others are refused.
+// 1 ReLU, 2 SiLU, 3 GELU in its tanh form, 4 GELU in its exact (erf) form, 5 the square of ReLU; others are refused.
 int st_gemm(void* out, const void* x, const void* w, const float* bias, const float* residual,
             int M, int N, int K, int activation, int dtype, int out_f32, int algo,
             const StGemmExtras* extras, hipStream_t stream);
@@ -99,15 +99,61 @@ int st_sample(int* out, const float* logits, int num_rows, int vocab, const floa
 float st_hash_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t draw, uint32_t v);
 
 // ---- short causal convolution over time, one filter a channel (csrc/token_conv.hip)
-// out[t, c] = x[t, c] + sum_j w[c, j] * x(row of position p_t - taps + 1 + j, c): rows before the
-// item's first row of this step come from state[slot, taps - 1, channels] (the inputs at the last
-// taps - 1 positions before it; zeros before the sequence's start).  st_token_conv_state then moves
+// out[t, c] = act((x[t, c] if add_input) + bias[c] + sum_j w[c, j] * x(row of position p_t - taps + 1 + j, c)):
+// x rows float or bfloat16 with stride x_stride; rows before the item's first row of this step come from
+// state + slot * slot_stride, [taps - 1, channels] floats (the inputs at the last taps - 1 positions
+// before it; zeros before the sequence's start).  st_token_conv_state then moves
 // the state on by the step's rows.  Rows whose item is -1 are written as zeros.
-int st_token_conv(void* out, const float* x, const float* w, const float* state, const int* token_item,
-                  const int* item_tok_off, const int* item_slot, int num_tokens, int channels, int taps,
-                  int add_input, int out_dtype, hipStream_t stream);
-int st_token_conv_state(float* state, const float* x, const int* item_len, const int* item_tok_off,
-                        const int* item_slot, int num_items, int channels, int taps, hipStream_t stream);
+int st_token_conv(void* out, const void* x, int64_t x_stride, int in_dtype, const float* w, const float* bias,
+                  const float* state, int64_t slot_stride, const int* token_item, const int* item_tok_off,
+                  const int* item_slot, int num_tokens, int channels, int taps, int add_input, int activation,
+                  int out_dtype, hipStream_t stream);
+int st_token_conv_state(float* state, int64_t slot_stride, const void* x, int64_t x_stride, int in_dtype,
+                        const int* item_len, const int* item_tok_off, const int* item_slot, int num_items,
+                        int channels, int taps, hipStream_t stream);
+
+// ---- rotary positions, one-pool page write, two float rows side by side in the storage type (csrc/rotary.hip)
+// In place on the rows' queries and keys: the first rot_dims coordinates of every head, coordinate i
+// paired with i + rot_dims / 2, turned by positions[t] * freq[i]; cosine and sine times `mult`.
+int st_rotary(void* q, int64_t q_stride, int q_heads, void* k, int64_t k_stride, int k_heads, int head_dim,
+              int rot_dims, const float* freq, float mult, const int* positions, int num_tokens, int dtype,
+              hipStream_t stream);
+// src[t, head, :] -> the token's entry of a pool [pages, heads, page_size, head_dim]; norm != 0: divided
+// by its root mean square over head_dim (eps inside the root) on the way.
+int st_paged_write(void* cache, int64_t page_stride, const void* src, int64_t src_stride, const int* token_item,
+                   const int* positions, const int* block_table, int max_pages, int page_size, int num_tokens,
+                   int heads, int head_dim, int norm, float eps, int dtype, hipStream_t stream);
+int st_concat_cast(void* out, const float* a, int wa, const float* b, int wb, int num_rows, int dtype,
+                   hipStream_t stream);
+
+// ---- attention with heads coupled before the softmax, a sink and a window (csrc/sink_attention.hip)
+int64_t st_sink_attention_lds(int heads, int key_dim, int mixed);
+int st_sink_attention(void* out, float* part_o, float* part_ml, const void* q, int64_t q_stride,
+                      const void* k_cache, int64_t k_page_stride, const void* v_cache, int64_t v_page_stride,
+                      const float* mix, const int* token_item, const int* positions, const int* block_table,
+                      int max_pages, int page_size, int num_tokens, int heads, int kv_heads, int key_dim,
+                      int value_dim, float scale, int window, int sink, int splits, int dtype, hipStream_t stream);
+
+// ---- recurrences with one decay a head and token (csrc/state_scan.hip)
+// mode 0: out_a = softplus(raw + bias), out_b = exp(-exp(a_log) * out_a), raw [T, heads];
+// mode 1: out_a = sigmoid(raw[:, :heads]), out_b = exp(-exp(a_log) * softplus(raw[:, heads:] + bias)).
+int st_recurrence_gates(float* out_a, float* out_b, const float* raw, int64_t raw_stride, const float* a_log,
+                        const float* bias, int num_tokens, int heads, int mode, hipStream_t stream);
+// x[t, head, :] <- x / sqrt(sum x^2 + eps) * scale, in place on float rows.
+int st_unit_norm(float* x, int64_t stride, int num_tokens, int heads, int dim, float eps, float scale,
+                 hipStream_t stream);
+// mode 0: S <- b S + (a k) v^T, o = S^T q + skip v;  mode 1: S <- b S, u = a (v - S^T k), S <- S + k u^T,
+// o = S^T q.  a, b float [T, heads]; q, k float rows of qk_heads heads; state [slots](slot_stride)
+// [heads, key_dim, value_dim] float.
+int st_state_scan(float* out, const float* q, int64_t q_stride, const float* k, int64_t k_stride, const float* v,
+                  int64_t v_stride, const float* gate_a, const float* gate_b, const float* skip, float* state,
+                  int64_t slot_stride, const int* item_len, const int* item_tok_off, const int* item_slot,
+                  int num_items, int heads, int qk_heads, int key_dim, int value_dim, int mode, hipStream_t stream);
+// out = val * rsqrt(mean(val^2) + eps) * gain (* silu(gate) unless gate_first) over each of `groups`
+// parts of a row, val = o (* silu(gate) if gate_first); gain [width], or [groups * width] if gain_per_group.
+int st_gated_group_norm(void* out, const float* o, const void* gate, int64_t gate_stride, const float* gain,
+                        int num_tokens, int groups, int width, int gain_per_group, int gate_first, float eps,
+                        int dtype, hipStream_t stream);
 
 // ---- gated linear attention (csrc/recurrent.hip)
 // out = sigmoid(z)^(inv_tau) over n floats (out may be z).

@@ -145,7 +145,7 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
                        int out_f32, int algo, const StGemmExtras* extras, hipStream_t stream) {
     ST_CHECK(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     ST_CHECK(activation_known(activation), "gemm: activation %d has no kernel (0 none, 1 ReLU, 2 SiLU, "
-             "3 GELU in its tanh form, 4 GELU in its exact form)", activation);
+             "3 GELU in its tanh form, 4 GELU in its exact form, 5 ReLU squared)", activation);
     const int act = activation;
     StGemmExtras ex = {};
     if (extras) ex = *extras;

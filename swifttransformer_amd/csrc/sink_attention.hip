@@ -1,0 +1,272 @@
+// Attention over a paged cache whose heads are coupled before the softmax, with a sink and a
+// sliding window, and keys and values of different sizes:
+//
+//   r_g(i, j)  = scale * q_g(i) . k_c(g)(j)                  c(g) = g / (heads / kv_heads)
+//   s_h(i, j)  = sum_g M[h, g] r_g(i, j)                     (M null: s = r)
+//   p_h(i, j)  = exp(s_h(i, j)) / (sink + sum_j' exp(s_h(i, j')))      over max(0, i - window + 1) <= j' <= i
+//   o_h(i)     = sum_j p_h(i, j) v_c(h)(j)
+//
+// sink = 1 puts a key of score 0 and no value into every row's sum (its softmax starts from the
+// maximum 0 and the sum 1); sink = 0 is the ordinary softmax.  Scores, the mix, maxima, sums and
+// the weighted values are float.
+//
+// Because every head's score of a key needs all heads' products with that key, a workgroup owns
+// a query row with all its heads and walks the row's keys in blocks of 64: products of all heads
+// with the block (a lane a key), the mix, one softmax update a head (a wave a head, a lane a key),
+// then the weighted sum of the block's values (a thread a group of output coordinates).  Keys may
+// be split over several workgroups a row (`splits`); their partial results are merged by a second
+// kernel.
+#include "api.h"
+#include "common.h"
+
+namespace st {
+
+constexpr int kKeyBlock = 64;
+
+struct SinkAttnArgs {
+    void* out;                 // [T, heads * value_dim] storage type
+    float* part_o;             // [T, splits, heads * value_dim] and
+    float* part_ml;            // [T, splits, heads, 2] (maximum, sum) when splits > 1
+    const void* q; int64_t q_stride;
+    const void* k_cache; int64_t k_page_stride;
+    const void* v_cache; int64_t v_page_stride;
+    const float* mix;          // [heads, heads] or null
+    const int* token_item; const int* positions; const int* block_table;
+    int max_pages, page_size, heads, kv_heads, key_dim, value_dim, window, sink, splits;
+    float scale;
+};
+
+template <typename T>
+__device__ inline float dot_row(const float* __restrict__ qs, const T* __restrict__ kp, int dim) {
+    constexpr int V = Elem<T>::kVec;
+    float acc = 0.f;
+    if (dim % V == 0) {
+        for (int d = 0; d < dim; d += V) {
+            float kv[V];
+            Elem<T>::load_vec(kp + d, kv);
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc = fmaf(qs[d + i], kv[i], acc);
+        }
+    } else {
+        for (int d = 0; d < dim; ++d) acc = fmaf(qs[d], Elem<T>::load(kp + d), acc);
+    }
+    return acc;
+}
+
+template <typename T, int ACC>
+__global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
+    extern __shared__ float lds[];
+    const int H = a.heads, dk = a.key_dim, dv = a.value_dim, per = a.heads / a.kv_heads;
+    float* qs = lds;                               // [H * dk]
+    float* sraw = qs + H * dk;                     // [H * 64]
+    float* smix = sraw + H * kKeyBlock;            // [H * 64]
+    float* mix_s = smix + H * kKeyBlock;           // [H * H] (if mix)
+    float* m_s = mix_s + (a.mix ? H * H : 0);      // [H]
+    float* l_s = m_s + H;
+    float* al_s = l_s + H;
+    int* pg = (int*)(al_s + H);                    // [64] page of each key of the block
+    int* sl = pg + kKeyBlock;                      // [64] its place in the page
+    const int t = blockIdx.x, split = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int item = a.token_item[t], pos = a.positions[t];
+    const int width = H * dv;
+    T* out = (T*)a.out + (int64_t)t * width;
+    if (item < 0 || pos < 0) {                     // a padding row
+        if (a.splits == 1)
+            for (int e = tid; e < width; e += 256) Elem<T>::store(out + e, 0.f);
+        else if (tid < H) {
+            float* ml = a.part_ml + (((int64_t)t * a.splits + split) * H + tid) * 2;
+            ml[0] = -INFINITY; ml[1] = 0.f;
+        }
+        return;
+    }
+    const T* q = (const T*)a.q + (int64_t)t * a.q_stride;
+    for (int e = tid; e < H * dk; e += 256) qs[e] = Elem<T>::load(q + e);
+    if (a.mix) for (int e = tid; e < H * H; e += 256) mix_s[e] = a.mix[e];
+    const bool with_sink = a.sink && split == 0;   // the sink belongs to one split only
+    if (tid < H) { m_s[tid] = with_sink ? 0.f : -INFINITY; l_s[tid] = with_sink ? 1.f : 0.f; }
+    float o[ACC];
+#pragma unroll
+    for (int i = 0; i < ACC; ++i) o[i] = 0.f;
+    const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+    // this split's share of the row's key blocks
+    const int blocks = (pos - lo) / kKeyBlock + 1;
+    const int share = (blocks + a.splits - 1) / a.splits;
+    const int b0 = split * share, b1 = min(blocks, b0 + share);
+    const int* bt = a.block_table + (int64_t)item * a.max_pages;
+    const T* kc = (const T*)a.k_cache;
+    const T* vc = (const T*)a.v_cache;
+    for (int b = b0; b < b1; ++b) {
+        const int j0 = lo + b * kKeyBlock;
+        const int nk = min(kKeyBlock, pos - j0 + 1);
+        __syncthreads();                           // the block before is done with the shared lists
+        if (tid < kKeyBlock) {
+            int page = -1, place = 0;
+            if (tid < nk) {
+                const int j = j0 + tid, pi = j / a.page_size;
+                page = bt[pi];
+                place = j - pi * a.page_size;
+            }
+            pg[tid] = page;
+            sl[tid] = place;
+        }
+        __syncthreads();
+        for (int p = tid; p < H * kKeyBlock; p += 256) {
+            const int g = p >> 6, jj = p & 63;
+            float s = 0.f;
+            if (pg[jj] >= 0) {
+                const T* kp = kc + (int64_t)pg[jj] * a.k_page_stride + ((int64_t)(g / per) * a.page_size + sl[jj]) * dk;
+                s = dot_row<T>(qs + g * dk, kp, dk) * a.scale;
+            }
+            sraw[p] = s;
+        }
+        __syncthreads();
+        for (int p = tid; p < H * kKeyBlock; p += 256) {
+            const int h = p >> 6, jj = p & 63;
+            float s = -INFINITY;
+            if (pg[jj] >= 0) {
+                if (a.mix) {
+                    s = 0.f;
+                    for (int g = 0; g < H; ++g) s = fmaf(mix_s[h * H + g], sraw[g * kKeyBlock + jj], s);
+                } else {
+                    s = sraw[p];
+                }
+            }
+            smix[p] = s;
+        }
+        __syncthreads();
+        for (int h = wave; h < H; h += 4) {
+            const float s = smix[h * kKeyBlock + lane];
+            const float m_old = m_s[h];
+            const float m_new = fmaxf(m_old, wave_max(s));
+            const float p = (s == -INFINITY) ? 0.f : expf(s - m_new);
+            smix[h * kKeyBlock + lane] = p;
+            const float sum = wave_sum(p);
+            if (lane == 0) {
+                const float alpha = (m_old == -INFINITY) ? 0.f : expf(m_old - m_new);
+                al_s[h] = alpha;
+                l_s[h] = l_s[h] * alpha + sum;
+                m_s[h] = m_new;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < ACC; ++i) {
+            const int e = tid + 256 * i;
+            if (e >= width) break;
+            const int h = e / dv, d = e - h * dv;
+            const int64_t head_off = (int64_t)(h / per) * a.page_size;
+            float acc = o[i] * al_s[h];
+            const float* pw = smix + h * kKeyBlock;
+            for (int jj = 0; jj < nk; ++jj) {
+                if (pg[jj] < 0) continue;
+                const T* vp = vc + (int64_t)pg[jj] * a.v_page_stride + (head_off + sl[jj]) * dv + d;
+                acc = fmaf(pw[jj], Elem<T>::load(vp), acc);
+            }
+            o[i] = acc;
+        }
+    }
+    __syncthreads();
+    if (a.splits == 1) {
+#pragma unroll
+        for (int i = 0; i < ACC; ++i) {
+            const int e = tid + 256 * i;
+            if (e >= width) break;
+            const float l = l_s[e / dv];
+            Elem<T>::store(out + e, l > 0.f ? o[i] / l : 0.f);
+        }
+    } else {
+        float* po = a.part_o + ((int64_t)t * a.splits + split) * width;
+#pragma unroll
+        for (int i = 0; i < ACC; ++i) {
+            const int e = tid + 256 * i;
+            if (e >= width) break;
+            po[e] = o[i];
+        }
+        if (tid < H) {
+            float* ml = a.part_ml + (((int64_t)t * a.splits + split) * H + tid) * 2;
+            ml[0] = m_s[tid]; ml[1] = l_s[tid];
+        }
+    }
+}
+
+// out[t, h, :] = sum_s e^(m_s - m) o_s / sum_s e^(m_s - m) l_s over the splits of a row
+template <typename T>
+__global__ __launch_bounds__(256) void sink_attention_merge_kernel(
+    T* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits, int heads,
+    int value_dim) {
+    const int t = blockIdx.x;
+    const int width = heads * value_dim;
+    for (int e = threadIdx.x; e < width; e += 256) {
+        const int h = e / value_dim;
+        float m = -INFINITY;
+        for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(((int64_t)t * splits + s) * heads + h) * 2]);
+        float num = 0.f, den = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const float* ml = part_ml + (((int64_t)t * splits + s) * heads + h) * 2;
+            if (ml[0] == -INFINITY) continue;
+            const float w = expf(ml[0] - m);
+            num = fmaf(w, part_o[((int64_t)t * splits + s) * width + e], num);
+            den = fmaf(w, ml[1], den);
+        }
+        Elem<T>::store(out + (int64_t)t * width + e, den > 0.f ? num / den : 0.f);
+    }
+}
+
+template <typename T>
+static int launch_sink_attention(const SinkAttnArgs& a, int num_tokens, size_t lds_bytes, hipStream_t stream) {
+    const int per_thread = (a.heads * a.value_dim + 255) / 256;
+    const dim3 grid(num_tokens, a.splits);
+    if (per_thread <= 2) sink_attention_kernel<T, 2><<<grid, 256, lds_bytes, stream>>>(a);
+    else if (per_thread <= 4) sink_attention_kernel<T, 4><<<grid, 256, lds_bytes, stream>>>(a);
+    else if (per_thread <= 8) sink_attention_kernel<T, 8><<<grid, 256, lds_bytes, stream>>>(a);
+    else if (per_thread <= 16) sink_attention_kernel<T, 16><<<grid, 256, lds_bytes, stream>>>(a);
+    else sink_attention_kernel<T, 32><<<grid, 256, lds_bytes, stream>>>(a);
+    ST_LAUNCH_CHECK("sink_attention");
+    if (a.splits > 1) {
+        sink_attention_merge_kernel<T><<<num_tokens, 256, 0, stream>>>((T*)a.out, a.part_o, a.part_ml, a.splits,
+                                                                      a.heads, a.value_dim);
+        ST_LAUNCH_CHECK("sink_attention_merge");
+    }
+    return 0;
+}
+
+}  // namespace st
+
+using namespace st;
+
+// LDS bytes a workgroup of st_sink_attention needs (the host checks it against the device's limit)
+extern "C" int64_t st_sink_attention_lds(int heads, int key_dim, int mixed) {
+    return 4 * ((int64_t)heads * key_dim + 2 * (int64_t)heads * kKeyBlock + (mixed ? (int64_t)heads * heads : 0) +
+                3 * (int64_t)heads + 2 * kKeyBlock);
+}
+
+extern "C" int st_sink_attention(void* out, float* part_o, float* part_ml, const void* q, int64_t q_stride,
+                                 const void* k_cache, int64_t k_page_stride, const void* v_cache,
+                                 int64_t v_page_stride, const float* mix, const int* token_item, const int* positions,
+                                 const int* block_table, int max_pages, int page_size, int num_tokens, int heads,
+                                 int kv_heads, int key_dim, int value_dim, float scale, int window, int sink,
+                                 int splits, int dtype, hipStream_t stream) {
+    ST_CHECK(num_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && key_dim > 0 && value_dim > 0,
+             "sink_attention: bad sizes");
+    ST_CHECK(page_size > 0 && max_pages > 0 && window >= 0 && splits >= 1 && splits <= 65535, "sink_attention: bad sizes");
+    ST_CHECK(heads <= 256, "sink_attention: up to 256 heads, not %d", heads);
+    ST_CHECK(heads * value_dim <= 32 * 256, "sink_attention: heads x value size up to 8192, not %d", heads * value_dim);
+    const int64_t lds_bytes = st_sink_attention_lds(heads, key_dim, mix != nullptr);
+    ST_CHECK(lds_bytes <= 64 * 1024, "sink_attention: %lld bytes of LDS a row (heads x key size too large)",
+             (long long)lds_bytes);
+    if (num_tokens == 0) return 0;
+    ST_CHECK(out && q && k_cache && v_cache && token_item && positions && block_table, "sink_attention: null operand");
+    ST_CHECK(splits == 1 || (part_o && part_ml), "sink_attention: split keys need room for the partial results");
+    SinkAttnArgs a;
+    a.out = out; a.part_o = part_o; a.part_ml = part_ml; a.q = q; a.q_stride = q_stride;
+    a.k_cache = k_cache; a.k_page_stride = k_page_stride; a.v_cache = v_cache; a.v_page_stride = v_page_stride;
+    a.mix = mix; a.token_item = token_item; a.positions = positions; a.block_table = block_table;
+    a.max_pages = max_pages; a.page_size = page_size; a.heads = heads; a.kv_heads = kv_heads;
+    a.key_dim = key_dim; a.value_dim = value_dim; a.window = window; a.sink = sink; a.splits = splits;
+    a.scale = scale;
+    if (dtype == kF32) return launch_sink_attention<float>(a, num_tokens, (size_t)lds_bytes, stream);
+    if (dtype == kBF16) return launch_sink_attention<bf16_t>(a, num_tokens, (size_t)lds_bytes, stream);
+    ST_CHECK(false, "sink_attention: unknown dtype %d", dtype);
+    return 0;
+}

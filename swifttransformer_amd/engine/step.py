@@ -143,10 +143,11 @@ class ModelRunner:
         # (the run's logits were a tensor of their own; those of a recorded decode step live in the
         # arena, beside the head's input, for up to max_seqs rows)
         need = self.arena.peak + cache_param.max_seqs * (self.model.vocab_size * 4 + 256)
+        hold = self.arena.peak_hold
         del ctx, cache, manager
         torch.cuda.empty_cache()
-        self.arena.peak = 0
-        self.arena.resize(need + need // 16 + (1 << 16))
+        self.arena.peak = self.arena.peak_hold = 0
+        self.arena.resize(need + need // 16 + (1 << 16), hold + (1 << 12) if hold else 0)
 
     # ----------------------------------------------------------------- requests
     def admit(self, req_id: Hashable) -> None:
@@ -424,7 +425,8 @@ def pages_that_fit(model: DecoderModel, page_size: int, fraction: float, device)
         raise ValueError(f"gpu_mem_fraction is a share of the free memory in (0, 1], not {fraction}")
     free, _total = torch.cuda.mem_get_info(torch.device(device))
     elem = 2 if model.dtype == torch.bfloat16 else 4
-    per_page = sum((2 if need.values else 1) * need.num_kv_heads * need.head_dim * page_size * elem
+    per_page = sum(need.num_kv_heads * (need.head_dim + ((need.value_dim or need.head_dim) if need.values else 0))
+                   * page_size * elem
                    for need in model.cache_needs().values() if need.kind == "paged_kv")
     if per_page == 0:
         return 1

@@ -6,6 +6,7 @@ loader and ``initDummyWeight`` (src/csrc/model/gpt/gpt_weight.cc:235-326, :329-4
 from .decoder import DecoderModel
 from . import opt  # noqa: F401  (registers OPTForCausalLM)
 from . import zitupel  # noqa: F401  (registers Zitupel)
+from . import zimorax  # noqa: F401  (registers Zimorax)
 from .opt import build_opt_spec
 
 __all__ = ["DecoderModel", "build_opt_spec", "build_model", "load_model", "random_model"]

@@ -68,6 +68,7 @@ class DecoderModel:
             if hasattr(layer.mixer, "use_position"):
                 layer.mixer.use_position(self.position)
             self.layers.append(layer)
+        self.entries = [build_part("reentry", ps, H, dtype) for ps in getattr(spec, "entries", [])]
         self.final_norm = build_part("norm", spec.final_norm, H, dtype) if spec.final_norm else None
         self.head = build_part("head", spec.head, H, dtype)
         self.schedule = list(spec.schedule)
@@ -79,6 +80,7 @@ class DecoderModel:
         yield self.position
         for layer in self.layers:
             yield from layer.parts()
+        yield from self.entries
         if self.final_norm is not None:
             yield self.final_norm
         yield self.head
@@ -149,10 +151,16 @@ class DecoderModel:
             # the reference refuses to run before weights are loaded (gptop_base.cc:47-49)
             raise RuntimeError("load the weights before running the model")
         ctx.position = self.position
-        x32 = self.embedding.forward(ctx, self.position)
+        if self.entries:
+            with K.arena.held():     # read again by the runs that start from it: it lives until the step ends
+                first32 = x32 = self.embedding.forward(ctx, self.position)
+        else:
+            x32 = self.embedding.forward(ctx, self.position)
         for run, e in enumerate(self.schedule):
             layer = self.layers[e.layer]
             K.arena.next_bank()      # what this run of a layer makes may be read until the next one ends
+            if e.enter is not None:
+                x32 = self.entries[e.enter].forward(x32, first32, ctx)
             if layer.mixer_conv is not None:
                 x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write,
                                                 conv_cache=caches.get(conv_cache_id(run)))

@@ -12,7 +12,10 @@ of an allocator between steps.
 
 The rule this puts on parts: a tensor made during a layer may be read until the end of the
 next layer and no longer; what has to outlive that belongs in the cache manager's per-request
-state.  A part that allocates with ``torch.empty`` itself is untouched by all this.
+state.  A part that allocates with ``torch.empty`` itself is untouched by all this.  The one
+exception is what a model needs from a step's beginning to its end (an embedding that later
+layers read again): tensors made inside ``held()`` come from a third region that is only reset
+when the next step begins.
 
 ``measure`` mode runs a step through the ordinary allocator and records how much each bank
 would have needed; ``ModelRunner`` uses it once, on a step of ``max_batched_tokens`` padding
@@ -42,26 +45,35 @@ class StepArena:
         self.peak = 0               # largest bank use seen (in measure mode: what a bank would have needed)
         self.overflows = 0          # requests served by the ordinary allocator because the bank was full
         self.carved = 0             # requests served from the buffer
+        self.hold_bytes = 0         # the region of tensors that live until the step ends
+        self.hold_used = 0
+        self.peak_hold = 0
+        self.holding = False        # True inside ``held()``: requests go to that region
 
-    def resize(self, bank_bytes: int) -> None:
-        """(Re)allocate the buffer: two banks of ``bank_bytes``.  Only before any step has been
-        recorded against it: recorded steps keep the addresses they were recorded with."""
+    def resize(self, bank_bytes: int, hold_bytes: int = 0) -> None:
+        """(Re)allocate the buffer: two banks of ``bank_bytes`` and ``hold_bytes`` for what lives
+        until the step ends.  Only before any step has been recorded against it: recorded steps
+        keep the addresses they were recorded with."""
         bank_bytes = -(-int(bank_bytes) // _ALIGN) * _ALIGN
+        hold_bytes = -(-int(hold_bytes) // _ALIGN) * _ALIGN
         self.bank_bytes = bank_bytes
+        self.hold_bytes = hold_bytes
         self._typed = {}
-        self.buffer = torch.empty(2 * bank_bytes, dtype=torch.uint8, device=self.device) if bank_bytes else None
+        total = 2 * bank_bytes + hold_bytes
+        self.buffer = torch.empty(total, dtype=torch.uint8, device=self.device) if total else None
         self.begin_step()
 
     def nbytes(self) -> int:
-        return 2 * self.bank_bytes
+        return 2 * self.bank_bytes + self.hold_bytes
 
     def begin_step(self) -> None:
         self.bank = 1               # the embedding's output; the first layer then starts bank 0
         self.used = [0, 0]
+        self.hold_used = 0
 
     def state(self):
         """Where the bump pointers stand (to go on from there later, see ``using``)."""
-        return (self.bank, tuple(self.used))
+        return (self.bank, tuple(self.used), self.hold_used)
 
     def next_bank(self) -> None:
         """A new layer starts: its tensors go to the other bank, from the bank's beginning."""
@@ -74,6 +86,22 @@ class StepArena:
             n *= int(d)
         size = _ITEMSIZE[dtype]
         nbytes = -(-(n * size) // _ALIGN) * _ALIGN
+        if self.holding:
+            off = self.hold_used
+            if self.measure or off + nbytes > self.hold_bytes:
+                if self.measure:
+                    self.hold_used = off + nbytes
+                    self.peak_hold = max(self.peak_hold, off + nbytes)
+                else:
+                    self.overflows += 1
+                return torch.empty(tuple(shape), dtype=dtype, device=self.device)
+            self.hold_used = off + nbytes
+            self.carved += 1
+            flat = self._typed.get(dtype)
+            if flat is None:
+                flat = self._typed[dtype] = self.buffer.view(dtype)
+            start = (2 * self.bank_bytes + off) // size
+            return flat[start:start + n].view(tuple(shape))
         off = self.used[self.bank]
         if self.measure or off + nbytes > self.bank_bytes:
             if self.measure:
@@ -126,10 +154,26 @@ def using(arena: Optional[StepArena], state=None):
             arena.begin_step()
         else:
             arena.bank, arena.used = state[0], list(state[1])
+            arena.hold_used = state[2] if len(state) > 2 else 0
     try:
         yield arena
     finally:
         _current = before
+
+
+@contextmanager
+def held():
+    """Inside: ``empty`` carves from the arena's region of tensors that live until the step ends
+    (no arena in use: the ordinary allocator, as always)."""
+    a = _current
+    before = a.holding if a is not None else False
+    if a is not None:
+        a.holding = True
+    try:
+        yield
+    finally:
+        if a is not None:
+            a.holding = before
 
 
 @contextmanager

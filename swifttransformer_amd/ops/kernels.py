@@ -65,9 +65,26 @@ def _lib():
         lib.st_probe_fill.argtypes = [_c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_p]
         lib.st_probe_mfma.argtypes = [_c_p, _c_int, _c_int, _c_int, _c_p]
         lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
-        lib.st_token_conv.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int,
-                                      _c_int, _c_p]
-        lib.st_token_conv_state.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_token_conv.argtypes = [_c_p, _c_p, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_int,
+                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
+        lib.st_token_conv_state.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_int, _c_p, _c_p, _c_p, _c_int, _c_int,
+                                            _c_int, _c_p]
+        lib.st_rotary.argtypes = [_c_p, _c_i64, _c_int, _c_p, _c_i64, _c_int, _c_int, _c_int, _c_p, _c_f, _c_p, _c_int,
+                                  _c_int, _c_p]
+        lib.st_paged_write.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int,
+                                       _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_concat_cast.argtypes = [_c_p, _c_p, _c_int, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_sink_attention_lds.restype = _c_i64
+        lib.st_sink_attention_lds.argtypes = [_c_int, _c_int, _c_int]
+        lib.st_sink_attention.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p,
+                                          _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int,
+                                          _c_int, _c_int, _c_int, _c_p]
+        lib.st_recurrence_gates.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_unit_norm.argtypes = [_c_p, _c_i64, _c_int, _c_int, _c_int, _c_f, _c_f, _c_p]
+        lib.st_state_scan.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_i64,
+                                      _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
+        lib.st_gated_group_norm.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                            _c_f, _c_int, _c_p]
         lib.st_decay_gate.argtypes = [_c_p, _c_p, _c_i64, _c_f, _c_p]
         lib.st_gla_scan.argtypes = [_c_p, _c_i64, _c_int, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p,
                                     _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_p]
@@ -341,7 +358,8 @@ def wide_offered(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
 
 # functions of the products' epilogues and of ``activation_multiply``, by the C interface's number
 # (csrc/activation.h; the names config files use for them)
-ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3, "gelu": 4, "gelu_erf": 4}
+ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3, "gelu": 4, "gelu_erf": 4,
+               "relu_squared": 5, "relu2": 5}
 
 
 def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_f32=False, algo=0,
@@ -726,34 +744,273 @@ def multiply(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = Non
 # ------------------------------------------------- short convolution over time
 def _d_token_conv(x, weight, state, ctx_arrays, out_dtype, **kw):
     n, c = x.shape
-    return {"rows": n, "width": c, "bytes": n * c * (4 + torch.empty((), dtype=out_dtype).element_size())}
+    return {"rows": n, "width": c, "bytes": n * c * (x.element_size() + torch.empty((), dtype=out_dtype).element_size())}
+
+
+def _slot_rows(state: torch.Tensor, name: str, inner: int) -> int:
+    """``state`` is [slots, ...] float with dense trailing dimensions of ``inner`` elements a slot (a whole
+    per-slot tensor, or a part of a larger one): the elements between slots."""
+    _need(state, name, torch.float32, contiguous=False)
+    if state[0].numel() != inner or not state[0].is_contiguous():
+        raise KernelError(f"{name}: a slot must hold {inner} dense floats")
+    return state.stride(0) if state.shape[0] > 1 else inner
 
 
 @_timed("token_conv", _d_token_conv)
 def token_conv(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx_arrays, out_dtype: torch.dtype,
-               add_input: bool = True, update_state: bool = True) -> torch.Tensor:
-    """y[t] = (x[t] if add_input) + sum_j weight[:, j] * x(position of t - taps + 1 + j) per channel,
-    over the rows of a batch: what lies before an item's first row is read from ``state``
-    [slots, taps - 1, channels] (float), which is then moved on by the item's rows.
+               add_input: bool = True, update_state: bool = True, bias: Optional[torch.Tensor] = None,
+               activation: str = "none") -> torch.Tensor:
+    """y[t] = act((x[t] if add_input) + bias + sum_j weight[:, j] * x(position of t - taps + 1 + j)) per
+    channel, over the rows of a batch: what lies before an item's first row is read from ``state``
+    [slots, taps - 1, channels] (float; the slots may be parts of a larger per-slot state), which is then
+    moved on by the item's rows.
 
-    x: float [T, channels]; weight: float [channels, taps]; ``ctx_arrays``: the batch's
-    (token_item, item_len, item_tok_off, item_slot)."""
+    x: float or bfloat16 [T, channels] (dense rows, any row stride); weight: float [channels, taps];
+    bias: float [channels] or None; ``ctx_arrays``: the batch's (token_item, item_len, item_tok_off,
+    item_slot)."""
     token_item, item_len, item_tok_off, item_slot = ctx_arrays
     T, C = x.shape
     taps = weight.shape[1]
-    _need(x, "x", torch.float32, (T, C))
+    _need(x, "x", None, (T, C), contiguous=False)
+    if x.stride(1) != 1:
+        raise KernelError("x: rows must be dense")
     _need(weight, "weight", torch.float32, (C, taps))
-    _need(state, "state", torch.float32, (state.shape[0], max(taps - 1, 0), C))
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (C,))
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"the kernels know the activations {sorted(ACTIVATIONS)}, not {activation!r}")
+    slot_stride = _slot_rows(state, "state", max(taps - 1, 0) * C) if taps > 1 else 0
     _need(token_item, "token_item", torch.int32, (T,))
     B = item_slot.shape[0]
     for name, v in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
         _need(v, name, torch.int32, (B,))
     out = empty((T, C), out_dtype, x.device)
-    _check(_lib().st_token_conv(_ptr(out), _ptr(x), _ptr(weight), _ptr(state), _ptr(token_item), _ptr(item_tok_off),
-                                _ptr(item_slot), T, C, taps, int(bool(add_input)), dtype_code(out_dtype), _stream()))
+    xs = x.stride(0) if T > 1 else C
+    _check(_lib().st_token_conv(_ptr(out), _ptr(x), xs, dtype_code(x.dtype), _ptr(weight), _ptr(bias), _ptr(state),
+                                slot_stride, _ptr(token_item), _ptr(item_tok_off), _ptr(item_slot), T, C, taps,
+                                int(bool(add_input)), ACTIVATIONS[activation], dtype_code(out_dtype), _stream()))
     if update_state:
-        _check(_lib().st_token_conv_state(_ptr(state), _ptr(x), _ptr(item_len), _ptr(item_tok_off), _ptr(item_slot),
-                                          B, C, taps, _stream()))
+        _check(_lib().st_token_conv_state(_ptr(state), slot_stride, _ptr(x), xs, dtype_code(x.dtype), _ptr(item_len),
+                                          _ptr(item_tok_off), _ptr(item_slot), B, C, taps, _stream()))
+    return out
+
+
+# ------------------------------------------- rotary positions, one-pool page write
+@_timed("rotary", lambda q, k, *a, **kw: {"rows": q.shape[0], "width": q.shape[1] + k.shape[1],
+                                          "bytes": 2 * q.shape[0] * (q.shape[1] + k.shape[1]) * q.element_size()})
+def rotary(q: torch.Tensor, k: torch.Tensor, head_dim: int, freq: torch.Tensor, mult: float,
+           positions: torch.Tensor) -> None:
+    """In place on q [T, heads * head_dim] and k [T, kv_heads * head_dim] (dense rows, any row stride): of
+    every head the first 2 * len(freq) coordinates are turned, coordinate i paired with i + len(freq), by
+    the angle positions[t] * freq[i]; cosine and sine are multiplied by ``mult``.  Rows with a negative
+    position are left alone."""
+    T = q.shape[0]
+    half = freq.shape[0]
+    _need(freq, "freq", torch.float32, (half,))
+    _need(positions, "positions", torch.int32, (T,))
+    for name, t in (("q", q), ("k", k)):
+        _need(t, name, q.dtype, (T, t.shape[1]), contiguous=False)
+        if t.stride(1) != 1 or t.shape[1] % head_dim:
+            raise KernelError(f"{name}: dense rows of whole heads")
+    if 2 * half > head_dim:
+        raise KernelError(f"{2 * half} turned coordinates do not fit a head of {head_dim}")
+    _check(_lib().st_rotary(_ptr(q), q.stride(0), q.shape[1] // head_dim, _ptr(k), k.stride(0), k.shape[1] // head_dim,
+                            head_dim, 2 * half, _ptr(freq), float(mult), _ptr(positions), T, dtype_code(q.dtype),
+                            _stream()))
+
+
+@_timed("paged_write", lambda cache, src, *a, **kw: {"rows": src.shape[0], "width": src.shape[1],
+                                                      "bytes": 2 * src.numel() * src.element_size()})
+def paged_write(cache: torch.Tensor, src: torch.Tensor, token_item: torch.Tensor, positions: torch.Tensor,
+                block_table: torch.Tensor, unit_eps: Optional[float] = None) -> None:
+    """Each row of src [T, heads * head_dim] (dense rows, any stride) becomes its token's entry of ``cache``
+    [pages, heads, page_size, head_dim]; with ``unit_eps`` every head's vector is divided by its root mean
+    square (eps inside the root) on the way, in float."""
+    num_pages, heads, ps, hd = cache.shape
+    T = src.shape[0]
+    _need(cache, "cache", src.dtype, (num_pages, heads, ps, hd), contiguous=False)
+    if cache.stride()[1:] != (ps * hd, hd, 1):
+        raise KernelError("cache: a page must be contiguous")
+    _need(src, "src", None, (T, heads * hd), contiguous=False)
+    if src.stride(1) != 1:
+        raise KernelError("src: rows must be dense")
+    _need(token_item, "token_item", torch.int32, (T,))
+    _need(positions, "positions", torch.int32, (T,))
+    _need(block_table, "block_table", torch.int32)
+    _check(_lib().st_paged_write(_ptr(cache), cache.stride(0), _ptr(src), src.stride(0), _ptr(token_item),
+                                 _ptr(positions), _ptr(block_table), block_table.shape[1], ps, T, heads, hd,
+                                 int(unit_eps is not None), float(unit_eps or 0.0), dtype_code(src.dtype), _stream()))
+
+
+@_timed("concat_cast", lambda a, b, dtype: {"rows": a.shape[0], "width": a.shape[1] + b.shape[1],
+                                            "bytes": (a.numel() + b.numel()) * (4 + torch.empty((), dtype=dtype).element_size())})
+def concat_cast(a: torch.Tensor, b: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """[a | b] row by row in ``dtype``, from float rows."""
+    T = a.shape[0]
+    _need(a, "a", torch.float32, (T, a.shape[1]))
+    _need(b, "b", torch.float32, (T, b.shape[1]))
+    out = empty((T, a.shape[1] + b.shape[1]), dtype, a.device)
+    _check(_lib().st_concat_cast(_ptr(out), _ptr(a), a.shape[1], _ptr(b), b.shape[1], T, dtype_code(dtype), _stream()))
+    return out
+
+
+# ------------------- attention with coupled heads, a sink and a window
+def sink_attention_fits(heads: int, key_dim: int, value_dim: int, mixed: bool) -> bool:
+    """Whether ``sink_attention`` takes these sizes (a row's queries and a block's scores live in LDS)."""
+    return (heads <= 256 and heads * value_dim <= 8192 and
+            int(_lib().st_sink_attention_lds(heads, key_dim, int(mixed))) <= 64 * 1024)
+
+
+def _d_sink_attention(q, k_cache, v_cache, token_item, positions, block_table, heads, scale, **kw):
+    return {"rows": q.shape[0], "heads": heads, "kv_heads": k_cache.shape[1], "head_dim": k_cache.shape[3],
+            "value_dim": v_cache.shape[3], "window": kw.get("window", 0), "splits": kw.get("num_splits", 1),
+            "elem": k_cache.element_size()}
+
+
+@_timed("sink_attention", _d_sink_attention)
+def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, token_item: torch.Tensor,
+                   positions: torch.Tensor, block_table: torch.Tensor, heads: int, scale: float, *,
+                   window: int = 0, sink: bool = True, head_mix: Optional[torch.Tensor] = None,
+                   num_splits: int = 1, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Each query row attends over its request's cached keys [max(0, p - window + 1), p] (window 0: from
+    0).  Every head's scaled products with a key are mixed over the heads by ``head_mix`` (float
+    [heads, heads], row = receiving head; None: no mix) before the softmax; ``sink``: one is added to the
+    softmax's denominator.
+
+    q: [T, heads * key_dim] (dense rows, any stride); k_cache [pages, kv_heads, page, key_dim];
+    v_cache [pages, kv_heads, page, value_dim].  Returns [T, heads * value_dim]."""
+    num_pages, nkv, ps, dk = k_cache.shape
+    dv = v_cache.shape[3]
+    T = q.shape[0]
+    _need(k_cache, "k_cache", q.dtype, (num_pages, nkv, ps, dk), contiguous=False)
+    _need(v_cache, "v_cache", q.dtype, (v_cache.shape[0], nkv, ps, dv), contiguous=False)
+    if k_cache.stride()[1:] != (ps * dk, dk, 1) or v_cache.stride()[1:] != (ps * dv, dv, 1):
+        raise KernelError("a page must be contiguous")
+    _need(q, "q", None, (T, heads * dk), contiguous=False)
+    if q.stride(1) != 1:
+        raise KernelError("q rows must be dense")
+    _need(token_item, "token_item", torch.int32, (T,))
+    _need(positions, "positions", torch.int32, (T,))
+    _need(block_table, "block_table", torch.int32)
+    if head_mix is not None:
+        _need(head_mix, "head_mix", torch.float32, (heads, heads))
+    if out is None:
+        out = empty((T, heads * dv), q.dtype, q.device)
+    _need(out, "out", q.dtype, (T, heads * dv))
+    part_o = part_ml = None
+    if num_splits > 1:
+        part_o = empty((T, num_splits, heads * dv), torch.float32, q.device)
+        part_ml = empty((T, num_splits, heads, 2), torch.float32, q.device)
+    _check(_lib().st_sink_attention(_ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(q), q.stride(0), _ptr(k_cache),
+                                    k_cache.stride(0), _ptr(v_cache), v_cache.stride(0), _ptr(head_mix),
+                                    _ptr(token_item), _ptr(positions), _ptr(block_table), block_table.shape[1], ps, T,
+                                    heads, nkv, dk, dv, float(scale), int(window), int(bool(sink)), int(num_splits),
+                                    dtype_code(q.dtype), _stream()))
+    return out
+
+
+# --------------------------------- recurrences with one decay a head and token
+def recurrence_gates(raw: torch.Tensor, a_log: torch.Tensor, bias: torch.Tensor, heads: int, mode: str):
+    """Two float [T, heads] tensors from float logits ``raw`` (dense rows, any stride):
+    ``"step"``: raw [T, heads] -> (step = softplus(raw + bias), decay = exp(-exp(a_log) * step));
+    ``"write"``: raw [T, 2 * heads] -> (strength = sigmoid(raw[:, :heads]),
+    decay = exp(-exp(a_log) * softplus(raw[:, heads:] + bias)))."""
+    T = raw.shape[0]
+    code = {"step": 0, "write": 1}[mode]
+    _need(raw, "raw", torch.float32, (T, heads * (1 + code)), contiguous=False)
+    if raw.stride(1) != 1:
+        raise KernelError("raw: rows must be dense")
+    _need(a_log, "a_log", torch.float32, (heads,))
+    _need(bias, "bias", torch.float32, (heads,))
+    a = empty((T, heads), torch.float32, raw.device)
+    b = empty((T, heads), torch.float32, raw.device)
+    _check(_lib().st_recurrence_gates(_ptr(a), _ptr(b), _ptr(raw), raw.stride(0), _ptr(a_log), _ptr(bias), T, heads,
+                                      code, _stream()))
+    return a, b
+
+
+def unit_norm(x: torch.Tensor, heads: int, eps: float, scale: float = 1.0) -> torch.Tensor:
+    """In place on float x [T, heads * dim] (dense rows, any stride): every head's vector divided by
+    sqrt(sum of its squares + eps) and multiplied by ``scale``."""
+    T = x.shape[0]
+    _need(x, "x", torch.float32, (T, x.shape[1]), contiguous=False)
+    if x.stride(1) != 1 or x.shape[1] % heads:
+        raise KernelError("x: dense rows of whole heads")
+    _check(_lib().st_unit_norm(_ptr(x), x.stride(0), T, heads, x.shape[1] // heads, float(eps), float(scale), _stream()))
+    return x
+
+
+def _d_state_scan(q, k, v, gate_a, gate_b, state, ctx_arrays, heads, mode, skip=None):
+    T = q.shape[0]
+    vd = v.shape[1] // heads
+    kd = state.shape[2]
+    return {"rows": T, "heads": heads, "key_dim": kd, "value_dim": vd, "items": ctx_arrays[2].shape[0],
+            "flops": (4 if mode == "additive" else 6) * T * heads * kd * vd,
+            "bytes": 4 * T * (q.shape[1] + k.shape[1] + 2 * v.shape[1] + 2 * heads) +
+                     8 * ctx_arrays[2].shape[0] * heads * kd * vd}
+
+
+@_timed("state_scan", _d_state_scan)
+def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate_a: torch.Tensor, gate_b: torch.Tensor,
+               state: torch.Tensor, ctx_arrays, heads: int, mode: str, skip: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Per item and head, from the slot's state S [key_dim, value_dim] and over the item's rows in order
+    (a = gate_a[t, head], b = gate_b[t, head]):
+    ``"additive"``: S <- b S + (a k_t) v_t^T, o_t = S^T q_t + skip[head] v_t;
+    ``"delta"``: S <- b S, u = a (v_t - S^T k_t), S <- S + k_t u^T, o_t = S^T q_t.
+    The state is stored back.  q, k: float [T, qk_heads * key_dim], v: float [T, heads * value_dim] (dense
+    rows, any stride; head h reads q/k head h // (heads / qk_heads)); state: float
+    [slots, heads, key_dim, value_dim] (slots may be parts of a larger per-slot state).  Returns float
+    [T, heads * value_dim]."""
+    _token_item, item_len, item_tok_off, item_slot = ctx_arrays
+    T = q.shape[0]
+    _, sh, kd, vd = state.shape
+    if sh != heads or v.shape[1] != heads * vd or q.shape[1] % kd or q.shape[1] != k.shape[1]:
+        raise KernelError("state_scan: the operands' sizes do not fit the state")
+    qk_heads = q.shape[1] // kd
+    if heads % qk_heads:
+        raise KernelError(f"{heads} heads do not divide over {qk_heads} query/key heads")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _need(t, name, torch.float32, (T, t.shape[1]), contiguous=False)
+        if t.stride(1) != 1:
+            raise KernelError(f"{name}: rows must be dense")
+    _need(gate_a, "gate_a", torch.float32, (T, heads))
+    _need(gate_b, "gate_b", torch.float32, (T, heads))
+    if skip is not None:
+        _need(skip, "skip", torch.float32, (heads,))
+    slot_stride = _slot_rows(state, "state", heads * kd * vd)
+    B = item_slot.shape[0]
+    for name, t in (("item_len", item_len), ("item_tok_off", item_tok_off), ("item_slot", item_slot)):
+        _need(t, name, torch.int32, (B,))
+    out = empty((T, heads * vd), torch.float32, q.device)
+    _check(_lib().st_state_scan(_ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
+                                _ptr(gate_a), _ptr(gate_b), _ptr(skip), _ptr(state), slot_stride, _ptr(item_len),
+                                _ptr(item_tok_off), _ptr(item_slot), B, heads, qk_heads, kd, vd,
+                                {"additive": 0, "delta": 1}[mode], _stream()))
+    return out
+
+
+@_timed("gated_group_norm", lambda o, gate, *a, **k: {"rows": o.shape[0], "width": o.shape[1],
+                                                       "bytes": o.numel() * (4 + 3 * gate.element_size())})
+def gated_group_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, groups: int, eps: float,
+                     out_dtype: torch.dtype, gate_first: bool = False) -> torch.Tensor:
+    """Each of the ``groups`` equal parts of a row of o (float [T, W]) divided by its root mean square and
+    multiplied by ``gain`` (float [W / groups] shared by the parts, or [W]) and by silu(gate) (``gate``:
+    [T, W] rows of ``out_dtype``, any stride); ``gate_first``: the gate multiplies before the norm."""
+    T, W = o.shape
+    if W % groups:
+        raise KernelError(f"{W} channels do not divide into {groups} parts")
+    width = W // groups
+    _need(o, "o", torch.float32, (T, W))
+    _need(gate, "gate", out_dtype, (T, W), contiguous=False)
+    if gate.stride(1) != 1:
+        raise KernelError("gate: rows must be dense")
+    if tuple(gain.shape) not in ((width,), (W,)):
+        raise KernelError(f"gain must have {width} or {W} entries")
+    _need(gain, "gain", torch.float32)
+    out = empty((T, W), out_dtype, o.device)
+    _check(_lib().st_gated_group_norm(_ptr(out), _ptr(o), _ptr(gate), gate.stride(0), _ptr(gain), T, groups, width,
+                                      int(gain.shape[0] == W and groups > 1), int(bool(gate_first)), float(eps),
+                                      dtype_code(out_dtype), _stream()))
     return out
 
 

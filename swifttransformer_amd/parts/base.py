@@ -28,6 +28,9 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
                 that has a ``mixer_conv`` part)
   token_conv    ``cache_need() -> CacheNeed``; ``forward(y32, ctx, cache) -> y_t``: a short causal
                 filter over time on what a mixer reads, with its last inputs as per-request state
+  reentry       ``forward(x32, first32, ctx) -> x32``: what happens to the residual stream before a run
+                of a layer that the schedule marks (``ScheduleEntry.enter``); ``first32`` is the
+                embedding's output of the step
 
 Any part may also offer ``step_planner() -> (key, planner)``: ``planner(items, info)`` sees the
 step's items on the host (slot, start, tokens of each) and a ``BatchInfo`` and returns a
@@ -48,7 +51,8 @@ import torch
 from ..weights.loader import TensorSpec
 from .spec import PartSpec
 
-CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "arrangement", "token_conv")
+CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "arrangement", "token_conv",
+              "reentry")
 _REGISTRY: Dict[str, Dict[str, Callable]] = {c: {} for c in CATEGORIES}
 
 
@@ -76,6 +80,7 @@ class CacheNeed:
     per token each; ``window`` > 0 means only the last ``window`` tokens are ever
     read, so pages behind it are given back.  ``values`` False: one vector per token serves as
     key and as value (a latent cache); no second pool is allocated and the view's ``v`` is its ``k``.
+    ``value_dim`` > 0: the values' heads have that size instead of ``head_dim``.
     kind "state": a fixed-size tensor per request (``state_shape``, ``state_dtype``),
     living in the request's state slot."""
     kind: str
@@ -85,10 +90,11 @@ class CacheNeed:
     state_shape: Tuple[int, ...] = ()
     state_dtype: Optional[torch.dtype] = None
     values: bool = True
+    value_dim: int = 0
 
     def group_key(self):
         return (self.kind, self.num_kv_heads, self.head_dim, self.window, self.state_shape,
-                self.state_dtype, self.values)
+                self.state_dtype, self.values, self.value_dim)
 
 
 @dataclass
@@ -149,6 +155,15 @@ class Part:
             return self.spec.names[logical]
         except KeyError:
             raise KeyError(f"{type(self).__name__}: spec names no tensor for {logical!r}") from None
+
+
+def fold_output_scale(weight: torch.Tensor, bias: Optional[torch.Tensor], scale: torch.Tensor):
+    """(diag(scale) W, scale * b): a per-feature factor on a product's result becomes part of its matrix
+    and bias (formed in float64, rounded once to the storage type), so that the product's epilogue can
+    add the residual as it always does."""
+    w = (weight.to(torch.float64) * scale.to(torch.float64)[:, None]).to(weight.dtype).contiguous()
+    b = None if bias is None else (bias.to(torch.float64) * scale.to(torch.float64)).to(bias.dtype).contiguous()
+    return w, b
 
 
 class Mixer(Part):

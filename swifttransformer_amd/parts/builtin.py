@@ -1,7 +1,7 @@
 """Registration of the parts that ship with the engine."""
 from .base import register_part
 from .norm import LayerNorm
-from .position import LearnedPositions, NoPositions
+from .position import LearnedPositions, NoPositions, RotaryPositions
 from .embedding import TokenEmbedding, LMHead
 from .feed_forward import DenseFeedForward
 from .attention import PagedAttention
@@ -10,6 +10,9 @@ from .conv import CausalTokenConv
 from .linear_attention import GatedLinearAttention
 from .latent_attention import LatentAttention
 from .routed import RoutedExperts
+from .sink_attention import SinkAttention
+from .state_space import Mamba2Mixer, GatedDeltaRule
+from .reentry import InputInjection
 
 register_part("norm", "layer_norm", LayerNorm)
 register_part("position", "learned", LearnedPositions)
@@ -24,3 +27,8 @@ register_part("token_conv", "causal", CausalTokenConv)
 register_part("mixer", "gated_linear_attention", GatedLinearAttention)
 register_part("mixer", "latent_attention", LatentAttention)
 register_part("feed_forward", "routed_experts", RoutedExperts)
+register_part("position", "rotary", RotaryPositions)
+register_part("mixer", "sink_attention", SinkAttention)
+register_part("mixer", "mamba2", Mamba2Mixer)
+register_part("mixer", "gated_delta", GatedDeltaRule)
+register_part("reentry", "input_injection", InputInjection)

@@ -12,13 +12,14 @@ import torch
 
 from ..ops import kernels as K
 from ..weights.loader import TensorSpec
-from .base import Part
+from .base import Part, fold_output_scale
 
 
 
 class DenseFeedForward(Part):
     """params: inner (int), activation (a name the products' epilogues know), bias (bool),
-    residual_scale (float, default 1: the factor with which the result enters the residual stream)."""
+    residual_scale (float, default 1: the factor with which the result enters the residual stream), out_scale
+    (bool: the file holds a per-feature factor on the result; it is folded into the second matrix and bias)."""
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
@@ -29,6 +30,7 @@ class DenseFeedForward(Part):
                              f"available: {sorted(K.ACTIVATIONS)}")
         self.bias = bool(self.param("bias", True))
         self.residual_scale = float(spec.params.get("residual_scale", 1.0))
+        self.out_scale = bool(spec.params.get("out_scale", False))
         self.w1 = self.b1 = self.w2 = self.b2 = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -38,6 +40,8 @@ class DenseFeedForward(Part):
         if self.bias:
             specs += [TensorSpec(self.name("fc1.bias"), (F,), "vector"),
                       TensorSpec(self.name("fc2.bias"), (H,), "vector")]
+        if self.out_scale:
+            specs.append(TensorSpec(self.name("out_scale"), (H,), "vector", init="gain"))
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
@@ -46,6 +50,8 @@ class DenseFeedForward(Part):
         if self.bias:
             self.b1 = tensors[self.name("fc1.bias")]
             self.b2 = tensors[self.name("fc2.bias")]
+        if self.out_scale:
+            self.w2, self.b2 = fold_output_scale(self.w2, self.b2, tensors[self.name("out_scale")])
 
     accepts_norm = True     # forward(..., norm=part) normalises residual32 itself
 

@@ -35,6 +35,7 @@ class ScheduleEntry:
     layer: int
     cache: int
     write: bool = True
+    enter: Optional[int] = None   # index into ``ModelSpec.entries``: that part acts on the stream before this run
 
 
 @dataclass
@@ -49,11 +50,16 @@ class ModelSpec:
     final_norm: Optional[PartSpec]
     head: PartSpec
     eos_token_id: Optional[int] = None
+    # parts of the category "reentry": what happens to the residual stream before the runs that name
+    # them (a pass over a group of layers that starts from a mix of the stream and the embedding)
+    entries: List[PartSpec] = field(default_factory=list)
 
     def validate(self) -> "ModelSpec":
         n = len(self.layers)
         written = set()
         for e in self.schedule:
+            if e.enter is not None and not 0 <= e.enter < len(self.entries):
+                raise ValueError(f"the schedule names entry {e.enter}; there are {len(self.entries)}")
             if not 0 <= e.layer < n:
                 raise ValueError(f"the schedule names layer {e.layer}; there are {n} layers")
             if e.write:

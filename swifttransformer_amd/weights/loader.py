@@ -31,7 +31,7 @@ class TensorSpec:
     kind: str = "matrix"            # matrix | table | vector | int
     optional: bool = False          # may be absent (e.g. a tied head)
     alt_names: Tuple[str, ...] = () # other spellings accepted in the file
-    init: str = "normal"            # random-weights mode: "normal" N(0, std) | "gain" 1 + N(0, 0.1)
+    init: str = "normal"            # random-weights mode: "normal" N(0, std) | "gain" 1 + N(0, 0.1) | "mix" I + N(0, 0.1)
 
 
 class WeightError(ValueError):

@@ -90,6 +90,8 @@ def random_tensor(spec: TensorSpec, seed: int, device="cpu") -> torch.Tensor:
     t = _standard_normal(n, _key_for(spec.name, seed), device).view(spec.shape)
     if spec.init == "gain":
         return t * GAIN_STD + 1.0
+    if spec.init == "mix":       # a square matrix near the identity
+        return t * GAIN_STD + torch.eye(spec.shape[0], spec.shape[1], dtype=t.dtype, device=t.device)
     return t * WEIGHT_STD
 
 
