@@ -247,3 +247,13 @@ def logits(cfg: dict, w: Dict[str, torch.Tensor], tokens) -> torch.Tensor:
     """float64 logits [T, vocab] of one sequence."""
     X = residual_streams(cfg, w, tokens)[-1]
     return layer_norm(X, w["final.norm"], float(cfg["norm"]["eps"])) @ w["head"].T
+
+
+def generate(cfg: dict, w: Dict[str, torch.Tensor], prompt, n: int) -> List[int]:
+    """Greedy continuation of ``prompt`` by ``n`` tokens (the lowest id on ties)."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        nxt = int(torch.argmax(logits(cfg, w, seq)[-1]))
+        out.append(nxt)
+        seq.append(nxt)
+    return out
