@@ -208,8 +208,8 @@ def kernel_times(args) -> int:
     return 0
 
 
-def side_by_side(args, shape: str) -> int:
-    """Zitupel beside OPT at the same layer sizes (width, heads, feed-forward width of OPT
+def side_by_side(args, shape: str, other: str = "zitupel") -> int:
+    """Another architecture (Zitupel, Zimorax) beside OPT at the same layer sizes (width, heads, feed-forward width of OPT
     ``shape``; the same number of layers, 8 unless ``--layers`` says otherwise; random weights):
     decode tokens/s at batch 1, 8 and 64 from 1,024-token prompts, a 2,048-token prefill, and for
     both the per-kernel times of one decode step at batch ``--batch`` and of the prefill with their
@@ -226,8 +226,8 @@ def side_by_side(args, shape: str) -> int:
     dt = parse_dtype(args.dtype)
     batch = args.batch
     out = {"shape": shape, "layers": layers, "dtype": args.dtype, "models": {}}
-    for family in ("zitupel", "opt"):
-        over = {"num_layers": layers} if family == "zitupel" else {"num_hidden_layers": layers}
+    for family in (other, "opt"):
+        over = {"num_layers": layers} if family != "opt" else {"num_hidden_layers": layers}
         hp = hyper_param_by_name(f"{family}_{shape}", **over)
         model = random_model(hp, dt, 0, "cuda:0")
         weights = sum(t.numel() * t.element_size() for p in model.all_parts() for t in vars(p).values()
@@ -254,14 +254,29 @@ def side_by_side(args, shape: str) -> int:
             runner.step([StepEntry(i, toks[i][:ctx_len], [])])
 
         def cost(keys_read, pairs):
+            def windowed(info):
+                # (keys read, query-key pairs) of a windowed attention: a decode row reads its window, a
+                # prompt's row i at most i + 1 keys; every key of a prompt is read at least once
+                w = info.get("window", 0)
+                if not w:
+                    return keys_read, pairs
+                if pairs == keys_read:                     # decode rows at a context of keys_read / rows
+                    seen = info["rows"] * min(w, keys_read // max(info["rows"], 1))
+                    return seen, seen
+                return keys_read, sum(min(i + 1, w) for i in range(keys_read))
+
             def nbytes(name, info):
                 if name in ("attention_rows", "attention_prefill"):
                     return 2 * keys_read * info["kv_heads"] * info["head_dim"] * info["elem"]
+                if name == "sink_attention":
+                    return windowed(info)[0] * info["kv_heads"] * (info["head_dim"] + info["value_dim"]) * info["elem"]
                 return None
 
             def flops(name, info):
                 if name in ("attention_rows", "attention_prefill"):
                     return 4.0 * pairs * info["heads"] * info["head_dim"]
+                if name == "sink_attention":
+                    return 2.0 * windowed(info)[1] * info["heads"] * (info["head_dim"] + info["value_dim"] + info["heads"])
                 return None
             return nbytes, flops
 
@@ -574,9 +589,10 @@ def main() -> int:
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     ap.add_argument("--workload", default="decode-1.3b",
                     choices=["decode-1.3b", "mixed-6.7b", "mixed-1.3b", "ttft", "decode-30b", "decode-family",
-                             "zitupel-125m", "zitupel-1.3b", "zitupel-6.7b"],
-                    help="decode-1.3b is the default line; the others are the other model shapes; zitupel-<size>: "
-                         "the Zitupel architecture beside OPT at the same layer sizes")
+                             "zitupel-125m", "zitupel-1.3b", "zitupel-6.7b",
+                             "zimorax-125m", "zimorax-1.3b", "zimorax-6.7b"],
+                    help="decode-1.3b is the default line; the others are the other model shapes; zitupel-<size>, "
+                         "zimorax-<size>: that architecture beside OPT at the same layer sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -599,8 +615,9 @@ def main() -> int:
         return decode_30b(args)
     if args.workload == "decode-family":
         return decode_family(args)
-    if args.workload.startswith("zitupel-"):
-        return side_by_side(args, args.workload.split("-", 1)[1])
+    if args.workload.startswith(("zitupel-", "zimorax-")):
+        family, shape = args.workload.split("-", 1)
+        return side_by_side(args, shape, family)
     steps = min(args.steps, CONTEXT - PROMPT_LEN)
     elem = 2 if args.dtype == "bf16" else 4
     biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)

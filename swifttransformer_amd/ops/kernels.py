@@ -910,6 +910,8 @@ def sink_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 
 
 # --------------------------------- recurrences with one decay a head and token
+@_timed("recurrence_gates", lambda raw, a_log, bias, heads, mode: {"rows": raw.shape[0], "width": heads,
+                                                                      "bytes": 4 * raw.shape[0] * (raw.shape[1] + 2 * heads)})
 def recurrence_gates(raw: torch.Tensor, a_log: torch.Tensor, bias: torch.Tensor, heads: int, mode: str):
     """Two float [T, heads] tensors from float logits ``raw`` (dense rows, any stride):
     ``"step"``: raw [T, heads] -> (step = softplus(raw + bias), decay = exp(-exp(a_log) * step));
@@ -929,6 +931,7 @@ def recurrence_gates(raw: torch.Tensor, a_log: torch.Tensor, bias: torch.Tensor,
     return a, b
 
 
+@_timed("unit_norm", lambda x, *a, **k: {"rows": x.shape[0], "width": x.shape[1], "bytes": 8 * x.numel()})
 def unit_norm(x: torch.Tensor, heads: int, eps: float, scale: float = 1.0) -> torch.Tensor:
     """In place on float x [T, heads * dim] (dense rows, any stride): every head's vector divided by
     sqrt(sum of its squares + eps) and multiplied by ``scale``."""
