@@ -36,27 +36,53 @@ struct SinkAttnArgs {
     float scale;
 };
 
-template <typename T>
-__device__ inline float dot_row(const float* __restrict__ qs, const T* __restrict__ kp, int dim) {
+// Products of up to four heads' queries (LDS, floats) with one key row: the row is loaded once, in
+// batches of four 16-byte pieces so that the loads are in flight together.
+template <typename T, int NQ>
+__device__ inline void dot_rows(const float* __restrict__ qs, int q_stride, const T* __restrict__ kp, int dim,
+                                float* acc) {
     constexpr int V = Elem<T>::kVec;
-    float acc = 0.f;
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) acc[n] = 0.f;
+    int d = 0;
     if (dim % V == 0) {
-        for (int d = 0; d < dim; d += V) {
+        for (; d + 4 * V <= dim; d += 4 * V) {
+            uint4 raw[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) raw[u] = *reinterpret_cast<const uint4*>(kp + d + u * V);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                float kv[V];
+                Elem<T>::unpack(raw[u], kv);
+#pragma unroll
+                for (int n = 0; n < NQ; ++n)
+#pragma unroll
+                    for (int i = 0; i < V; ++i) acc[n] = fmaf(qs[n * q_stride + d + u * V + i], kv[i], acc[n]);
+            }
+        }
+        for (; d < dim; d += V) {
             float kv[V];
             Elem<T>::load_vec(kp + d, kv);
 #pragma unroll
-            for (int i = 0; i < V; ++i) acc = fmaf(qs[d + i], kv[i], acc);
+            for (int n = 0; n < NQ; ++n)
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[n] = fmaf(qs[n * q_stride + d + i], kv[i], acc[n]);
         }
     } else {
-        for (int d = 0; d < dim; ++d) acc = fmaf(qs[d], Elem<T>::load(kp + d), acc);
+        for (; d < dim; ++d) {
+            const float kv = Elem<T>::load(kp + d);
+#pragma unroll
+            for (int n = 0; n < NQ; ++n) acc[n] = fmaf(qs[n * q_stride + d], kv, acc[n]);
+        }
     }
-    return acc;
 }
 
-template <typename T, int ACC>
+// NG groups of W neighbouring output coordinates a thread (W = 1, or the elements of a 16-byte load
+// where the value size is a multiple of that)
+template <typename T, int NG, int W>
 __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
     extern __shared__ float lds[];
-    const int H = a.heads, dk = a.key_dim, dv = a.value_dim, per = a.heads / a.kv_heads;
+    const int H = a.heads, G = a.kv_heads, dk = a.key_dim, dv = a.value_dim, per = a.heads / a.kv_heads;
     float* qs = lds;                               // [H * dk]
     float* sraw = qs + H * dk;                     // [H * 64]
     float* smix = sraw + H * kKeyBlock;            // [H * 64]
@@ -64,8 +90,10 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
     float* m_s = mix_s + (a.mix ? H * H : 0);      // [H]
     float* l_s = m_s + H;
     float* al_s = l_s + H;
-    int* pg = (int*)(al_s + H);                    // [64] page of each key of the block
-    int* sl = pg + kKeyBlock;                      // [64] its place in the page
+    // where each key of the block lies in the two pools (elements from the pool's start, before the
+    // head's share of the page); keys beyond the block's last repeat its first and weigh nothing
+    int64_t* koff = (int64_t*)(al_s + H + (((al_s + H) - lds) & 1));     // [64], 8-byte aligned
+    int64_t* voff = koff + kKeyBlock;                             // [64]
     const int t = blockIdx.x, split = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int item = a.token_item[t], pos = a.positions[t];
@@ -81,13 +109,22 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
         return;
     }
     const T* q = (const T*)a.q + (int64_t)t * a.q_stride;
-    for (int e = tid; e < H * dk; e += 256) qs[e] = Elem<T>::load(q + e);
+    for (int e = tid; e < H * dk; e += 256) qs[e] = Elem<T>::load(q + e) * a.scale;
     if (a.mix) for (int e = tid; e < H * H; e += 256) mix_s[e] = a.mix[e];
     const bool with_sink = a.sink && split == 0;   // the sink belongs to one split only
     if (tid < H) { m_s[tid] = with_sink ? 0.f : -INFINITY; l_s[tid] = with_sink ? 1.f : 0.f; }
-    float o[ACC];
+    // the output coordinates of this thread: head, and where its value channel lies within a key's values
+    // (a thread beyond the row's width repeats coordinate 0 and stores nothing)
+    float o[NG][W];
+    int oh[NG], ov[NG];
 #pragma unroll
-    for (int i = 0; i < ACC; ++i) o[i] = 0.f;
+    for (int i = 0; i < NG; ++i) {
+        const int e = (tid + 256 * i) * W < width ? (tid + 256 * i) * W : 0;
+#pragma unroll
+        for (int w = 0; w < W; ++w) o[i][w] = 0.f;
+        oh[i] = e / dv;
+        ov[i] = (oh[i] / per) * a.page_size * dv + (e - oh[i] * dv);
+    }
     const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
     // this split's share of the row's key blocks
     const int blocks = (pos - lo) / kKeyBlock + 1;
@@ -101,30 +138,34 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
         const int nk = min(kKeyBlock, pos - j0 + 1);
         __syncthreads();                           // the block before is done with the shared lists
         if (tid < kKeyBlock) {
-            int page = -1, place = 0;
-            if (tid < nk) {
-                const int j = j0 + tid, pi = j / a.page_size;
-                page = bt[pi];
-                place = j - pi * a.page_size;
-            }
-            pg[tid] = page;
-            sl[tid] = place;
+            const int j = j0 + (tid < nk ? tid : 0), pi = j / a.page_size;
+            const int page = max(bt[pi], 0);
+            const int place = j - pi * a.page_size;
+            koff[tid] = (int64_t)page * a.k_page_stride + (int64_t)place * dk;
+            voff[tid] = (int64_t)page * a.v_page_stride + (int64_t)place * dv;
         }
         __syncthreads();
-        for (int p = tid; p < H * kKeyBlock; p += 256) {
-            const int g = p >> 6, jj = p & 63;
-            float s = 0.f;
-            if (pg[jj] >= 0) {
-                const T* kp = kc + (int64_t)pg[jj] * a.k_page_stride + ((int64_t)(g / per) * a.page_size + sl[jj]) * dk;
-                s = dot_row<T>(qs + g * dk, kp, dk) * a.scale;
+        // a thread a (key head, key): the key row is loaded once for the heads that share it
+        for (int p = tid; p < G * kKeyBlock; p += 256) {
+            const int c = p >> 6, jj = p & 63;
+            const T* kp = kc + koff[jj] + (int64_t)c * a.page_size * dk;
+            for (int g0 = c * per; g0 < (c + 1) * per; g0 += 4) {
+                const int n = min(4, (c + 1) * per - g0);
+                float acc[4] = {0.f, 0.f, 0.f, 0.f};
+                if (n == 4) dot_rows<T, 4>(qs + g0 * dk, dk, kp, dk, acc);
+                else if (n == 3) dot_rows<T, 3>(qs + g0 * dk, dk, kp, dk, acc);
+                else if (n == 2) dot_rows<T, 2>(qs + g0 * dk, dk, kp, dk, acc);
+                else dot_rows<T, 1>(qs + g0 * dk, dk, kp, dk, acc);
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (u < n) sraw[(g0 + u) * kKeyBlock + jj] = acc[u];
             }
-            sraw[p] = s;
         }
         __syncthreads();
         for (int p = tid; p < H * kKeyBlock; p += 256) {
             const int h = p >> 6, jj = p & 63;
             float s = -INFINITY;
-            if (pg[jj] >= 0) {
+            if (jj < nk) {
                 if (a.mix) {
                     s = 0.f;
                     for (int g = 0; g < H; ++g) s = fmaf(mix_s[h * H + g], sraw[g * kKeyBlock + jj], s);
@@ -151,42 +192,52 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
         }
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < ACC; ++i) {
-            const int e = tid + 256 * i;
-            if (e >= width) break;
-            const int h = e / dv, d = e - h * dv;
-            const int64_t head_off = (int64_t)(h / per) * a.page_size;
-            float acc = o[i] * al_s[h];
-            const float* pw = smix + h * kKeyBlock;
-            for (int jj = 0; jj < nk; ++jj) {
-                if (pg[jj] < 0) continue;
-                const T* vp = vc + (int64_t)pg[jj] * a.v_page_stride + (head_off + sl[jj]) * dv + d;
-                acc = fmaf(pw[jj], Elem<T>::load(vp), acc);
+        for (int i = 0; i < NG; ++i) {
+            const float al = al_s[oh[i]];
+#pragma unroll
+            for (int w = 0; w < W; ++w) o[i][w] *= al;
+        }
+#pragma unroll 1
+        for (int jj = 0; jj < kKeyBlock; jj += 4) {              // loads of four keys in flight, then their sums
+            const int64_t v0 = voff[jj], v1 = voff[jj + 1], v2 = voff[jj + 2], v3 = voff[jj + 3];
+#pragma unroll
+            for (int i = 0; i < NG; ++i) {
+                const T* vh = vc + ov[i];
+                float x0[W], x1[W], x2[W], x3[W];
+                if (W == 1) {
+                    x0[0] = Elem<T>::load(vh + v0); x1[0] = Elem<T>::load(vh + v1);
+                    x2[0] = Elem<T>::load(vh + v2); x3[0] = Elem<T>::load(vh + v3);
+                } else {
+                    Elem<T>::load_vec(vh + v0, x0); Elem<T>::load_vec(vh + v1, x1);
+                    Elem<T>::load_vec(vh + v2, x2); Elem<T>::load_vec(vh + v3, x3);
+                }
+                const float* pw = smix + oh[i] * kKeyBlock + jj;
+                const float p0 = pw[0], p1 = pw[1], p2 = pw[2], p3 = pw[3];
+#pragma unroll
+                for (int w = 0; w < W; ++w)
+                    o[i][w] = fmaf(p3, x3[w], fmaf(p2, x2[w], fmaf(p1, x1[w], fmaf(p0, x0[w], o[i][w]))));
             }
-            o[i] = acc;
         }
     }
     __syncthreads();
-    if (a.splits == 1) {
+    float* po = a.splits == 1 ? nullptr : a.part_o + ((int64_t)t * a.splits + split) * width;
 #pragma unroll
-        for (int i = 0; i < ACC; ++i) {
-            const int e = tid + 256 * i;
-            if (e >= width) break;
-            const float l = l_s[e / dv];
-            Elem<T>::store(out + e, l > 0.f ? o[i] / l : 0.f);
-        }
-    } else {
-        float* po = a.part_o + ((int64_t)t * a.splits + split) * width;
+    for (int i = 0; i < NG; ++i) {
+        const int e = (tid + 256 * i) * W;
+        if (e >= width) break;
+        if (po) {
 #pragma unroll
-        for (int i = 0; i < ACC; ++i) {
-            const int e = tid + 256 * i;
-            if (e >= width) break;
-            po[e] = o[i];
+            for (int w = 0; w < W; ++w) po[e + w] = o[i][w];
+        } else {
+            const float l = l_s[oh[i]];
+            const float r = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+            for (int w = 0; w < W; ++w) Elem<T>::store(out + e + w, o[i][w] * r);
         }
-        if (tid < H) {
-            float* ml = a.part_ml + (((int64_t)t * a.splits + split) * H + tid) * 2;
-            ml[0] = m_s[tid]; ml[1] = l_s[tid];
-        }
+    }
+    if (po && tid < H) {
+        float* ml = a.part_ml + (((int64_t)t * a.splits + split) * H + tid) * 2;
+        ml[0] = m_s[tid]; ml[1] = l_s[tid];
     }
 }
 
@@ -195,33 +246,50 @@ template <typename T>
 __global__ __launch_bounds__(256) void sink_attention_merge_kernel(
     T* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits, int heads,
     int value_dim) {
+    __shared__ float wgt[256 * 16];                // [heads, splits]: a split's weight in its head's sum
     const int t = blockIdx.x;
     const int width = heads * value_dim;
-    for (int e = threadIdx.x; e < width; e += 256) {
-        const int h = e / value_dim;
+    const float* ml = part_ml + (int64_t)t * splits * heads * 2;
+    const float* po = part_o + (int64_t)t * splits * width;
+    for (int h = threadIdx.x; h < heads; h += 256) {
         float m = -INFINITY;
-        for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(((int64_t)t * splits + s) * heads + h) * 2]);
-        float num = 0.f, den = 0.f;
+        for (int s = 0; s < splits; ++s) m = fmaxf(m, ml[(s * heads + h) * 2]);
+        float den = 0.f;
         for (int s = 0; s < splits; ++s) {
-            const float* ml = part_ml + (((int64_t)t * splits + s) * heads + h) * 2;
-            if (ml[0] == -INFINITY) continue;
-            const float w = expf(ml[0] - m);
-            num = fmaf(w, part_o[((int64_t)t * splits + s) * width + e], num);
-            den = fmaf(w, ml[1], den);
+            const float ms = ml[(s * heads + h) * 2];
+            const float w = ms == -INFINITY ? 0.f : expf(ms - m);
+            wgt[h * splits + s] = w;
+            den = fmaf(w, ml[(s * heads + h) * 2 + 1], den);
         }
-        Elem<T>::store(out + (int64_t)t * width + e, den > 0.f ? num / den : 0.f);
+        const float r = den > 0.f ? 1.f / den : 0.f;
+        for (int s = 0; s < splits; ++s) wgt[h * splits + s] *= r;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < width; e += 256) {
+        const float* w = wgt + (e / value_dim) * splits;
+        float num = 0.f;
+        for (int s = 0; s < splits; ++s) num = fmaf(w[s], po[(int64_t)s * width + e], num);
+        Elem<T>::store(out + (int64_t)t * width + e, num);
     }
 }
 
 template <typename T>
 static int launch_sink_attention(const SinkAttnArgs& a, int num_tokens, size_t lds_bytes, hipStream_t stream) {
-    const int per_thread = (a.heads * a.value_dim + 255) / 256;
+    constexpr int V = Elem<T>::kVec;
+    const int width = a.heads * a.value_dim;
     const dim3 grid(num_tokens, a.splits);
-    if (per_thread <= 2) sink_attention_kernel<T, 2><<<grid, 256, lds_bytes, stream>>>(a);
-    else if (per_thread <= 4) sink_attention_kernel<T, 4><<<grid, 256, lds_bytes, stream>>>(a);
-    else if (per_thread <= 8) sink_attention_kernel<T, 8><<<grid, 256, lds_bytes, stream>>>(a);
-    else if (per_thread <= 16) sink_attention_kernel<T, 16><<<grid, 256, lds_bytes, stream>>>(a);
-    else sink_attention_kernel<T, 32><<<grid, 256, lds_bytes, stream>>>(a);
+    if (a.value_dim % V == 0) {
+        const int per_thread = (width / V + 255) / 256;
+        if (per_thread <= 1) sink_attention_kernel<T, 1, V><<<grid, 256, lds_bytes, stream>>>(a);
+        else if (per_thread <= 2) sink_attention_kernel<T, 2, V><<<grid, 256, lds_bytes, stream>>>(a);
+        else if (per_thread <= 4) sink_attention_kernel<T, 4, V><<<grid, 256, lds_bytes, stream>>>(a);
+        else sink_attention_kernel<T, 32 / V, V><<<grid, 256, lds_bytes, stream>>>(a);
+    } else {
+        const int per_thread = (width + 255) / 256;
+        if (per_thread <= 2) sink_attention_kernel<T, 2, 1><<<grid, 256, lds_bytes, stream>>>(a);
+        else if (per_thread <= 8) sink_attention_kernel<T, 8, 1><<<grid, 256, lds_bytes, stream>>>(a);
+        else sink_attention_kernel<T, 32, 1><<<grid, 256, lds_bytes, stream>>>(a);
+    }
     ST_LAUNCH_CHECK("sink_attention");
     if (a.splits > 1) {
         sink_attention_merge_kernel<T><<<num_tokens, 256, 0, stream>>>((T*)a.out, a.part_o, a.part_ml, a.splits,
@@ -238,7 +306,7 @@ using namespace st;
 // LDS bytes a workgroup of st_sink_attention needs (the host checks it against the device's limit)
 extern "C" int64_t st_sink_attention_lds(int heads, int key_dim, int mixed) {
     return 4 * ((int64_t)heads * key_dim + 2 * (int64_t)heads * kKeyBlock + (mixed ? (int64_t)heads * heads : 0) +
-                3 * (int64_t)heads + 2 * kKeyBlock);
+                3 * (int64_t)heads + 1 + 4 * kKeyBlock);
 }
 
 extern "C" int st_sink_attention(void* out, float* part_o, float* part_ml, const void* q, int64_t q_stride,
@@ -249,7 +317,7 @@ extern "C" int st_sink_attention(void* out, float* part_o, float* part_ml, const
                                  int splits, int dtype, hipStream_t stream) {
     ST_CHECK(num_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && key_dim > 0 && value_dim > 0,
              "sink_attention: bad sizes");
-    ST_CHECK(page_size > 0 && max_pages > 0 && window >= 0 && splits >= 1 && splits <= 65535, "sink_attention: bad sizes");
+    ST_CHECK(page_size > 0 && max_pages > 0 && window >= 0 && splits >= 1 && splits <= 16, "sink_attention: 1 to 16 splits");
     ST_CHECK(heads <= 256, "sink_attention: up to 256 heads, not %d", heads);
     ST_CHECK(heads * value_dim <= 32 * 256, "sink_attention: heads x value size up to 8192, not %d", heads * value_dim);
     const int64_t lds_bytes = st_sink_attention_lds(heads, key_dim, mix != nullptr);

@@ -13,8 +13,8 @@
 // Launch: a workgroup a (head, block of 64 value channels, item); lane = value channel, wave = a
 // part of 16 key channels, whose column of the state stays in registers.  The waves' partial dot
 // products meet in LDS: one barrier a token for the additive form, two for the delta rule (its
-// write needs S^T k over all key channels first).  The next token's operands are loaded before the
-// current one is used.
+// write needs S^T k over all key channels first).  Operands are staged through LDS a chunk of
+// tokens at a time.
 #include "api.h"
 #include "common.h"
 
@@ -62,18 +62,24 @@ __global__ __launch_bounds__(256) void unit_norm_kernel(float* __restrict__ x, i
     for (int j = lane; j < dim; j += 64) p[j] *= r;
 }
 
-template <int MODE>
-__global__ void state_scan_kernel(
+// Operands of `chunk` tokens at a time are staged in LDS, q [chunk, key_dim] | k [chunk, key_dim] |
+// v [chunk, 64] | a [chunk] | b [chunk], so that the walk over the tokens waits for LDS only.
+// floats a thread carries from memory to LDS for a chunk: what its register budget allows
+constexpr int scan_regs(int max_parts) { return max_parts >= 16 ? 6 : max_parts >= 8 ? 16 : 32; }
+
+template <int MODE, int MAXPARTS>
+__global__ __launch_bounds__(64 * MAXPARTS) void state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
     int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ ga,
     const float* __restrict__ gb, const float* __restrict__ skip, float* __restrict__ state, int64_t slot_stride,
     const int* __restrict__ item_len, const int* __restrict__ item_tok_off, const int* __restrict__ item_slot,
-    int heads, int qk_heads, int key_dim, int value_dim) {
+    int heads, int qk_heads, int key_dim, int value_dim, int chunk) {
+    extern __shared__ __attribute__((aligned(16))) float staged[];   // a chunk's operands, then its results [chunk, 64]
     __shared__ float red[2][kScanMaxParts][64];
     const int head = blockIdx.x, item = blockIdx.z;
-    const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
-    const int parts = blockDim.x >> 6;
-    const int col = blockIdx.y * 64 + lane;
+    const int tid = threadIdx.x, lane = tid & 63, part = tid >> 6;
+    const int nthreads = blockDim.x, parts = nthreads >> 6;
+    const int col0 = blockIdx.y * 64, col = col0 + lane;
     const bool live = col < value_dim;
     const int slot = item_slot[item], n = item_len[item];
     if (slot < 0 || n <= 0) return;                     // uniform over the workgroup
@@ -86,69 +92,111 @@ __global__ void state_scan_kernel(
     for (int i = 0; i < kScanPart; ++i)
         S[i] = (live && k0 + i < key_dim) ? sp[(int64_t)i * value_dim] : 0.f;
     const float d_skip = skip ? skip[head] : 0.f;
-    const float* qp = q + row0 * q_stride + (int64_t)qk_head * key_dim + k0;
-    const float* kp = k + row0 * k_stride + (int64_t)qk_head * key_dim + k0;
-    const float* vp = v + row0 * v_stride + (int64_t)head * value_dim + col;
+    const float* qp = q + row0 * q_stride + (int64_t)qk_head * key_dim;
+    const float* kp = k + row0 * k_stride + (int64_t)qk_head * key_dim;
+    const float* vp = v + row0 * v_stride + (int64_t)head * value_dim + col0;
     const float* ap = ga + row0 * heads + head;
     const float* bp = gb + row0 * heads + head;
-    float* op = out + row0 * ((int64_t)heads * value_dim) + (int64_t)head * value_dim + col;
-    float nq[kScanPart], nk[kScanPart], nv, na, nb;
-    auto fetch = [&](int t) {
+    float* op = out + row0 * ((int64_t)heads * value_dim) + (int64_t)head * value_dim + col0;
+    const int kdp = kScanPart * parts;                  // a row of q or k in LDS: padded with zeros to whole parts
+    const int nq = chunk * kdp, nv = chunk * 64;
+    // A chunk's operands go to LDS through registers: all of a thread's loads are issued before any is
+    // stored, so that a chunk costs one trip to memory, not one an element.  Rows beyond the item's end
+    // are zeros.
+    const int per_buf = 2 * nq + nv + 2 * chunk;
+    float* res = staged + per_buf;
+    const int chunks = (n + chunk - 1) / chunk;
+    for (int c = 0; c < chunks; ++c) {
+        const float* buf = staged;
+        const int t0 = c * chunk;
+        constexpr int kRegs = scan_regs(MAXPARTS);
+        float pre[kRegs];
 #pragma unroll
-        for (int i = 0; i < kScanPart; ++i) {
-            const bool in = k0 + i < key_dim;
-            nq[i] = in ? qp[(int64_t)t * q_stride + i] : 0.f;
-            nk[i] = in ? kp[(int64_t)t * k_stride + i] : 0.f;
+        for (int i = 0; i < kRegs; ++i) {
+            const int idx = tid + i * nthreads;
+            const float* src = nullptr;
+            if (idx < 2 * nq) {
+                const int j = idx < nq ? idx : idx - nq;
+                const int r = j / kdp, cc = j - r * kdp;
+                if (t0 + r < n && cc < key_dim) src = idx < nq ? qp + (int64_t)(t0 + r) * q_stride + cc : kp + (int64_t)(t0 + r) * k_stride + cc;
+            } else if (idx < 2 * nq + nv) {
+                const int j = idx - 2 * nq, r = j >> 6, cc = j & 63;
+                if (t0 + r < n && col0 + cc < value_dim) src = vp + (int64_t)(t0 + r) * v_stride + cc;
+            } else if (idx < per_buf) {
+                const int j = idx - 2 * nq - nv;
+                const int r = j < chunk ? j : j - chunk;
+                if (t0 + r < n) src = (j < chunk ? ap : bp) + (int64_t)(t0 + r) * heads;
+            }
+            pre[i] = src ? *src : 0.f;
         }
-        nv = live ? vp[(int64_t)t * v_stride] : 0.f;
-        na = ap[(int64_t)t * heads];
-        nb = bp[(int64_t)t * heads];
-    };
-    fetch(0);
-    for (int t = 0; t < n; ++t) {
-        float cq[kScanPart], ck[kScanPart];
+        __syncthreads();                     // the chunk before has been walked by every wave
 #pragma unroll
-        for (int i = 0; i < kScanPart; ++i) { cq[i] = nq[i]; ck[i] = nk[i]; }
-        const float cv = nv, ca = na, cb = nb;
-        if (t + 1 < n) fetch(t + 1);
-        float acc = 0.f;
-        if (MODE == 0) {
-            // ca: the step size, cb: the decay
-            const float w = ca * cv;
+        for (int i = 0; i < kRegs; ++i) {
+            const int idx = tid + i * nthreads;
+            if (idx < per_buf) staged[idx] = pre[i];
+        }
+        __syncthreads();
+        const int rows = min(chunk, n - c * chunk);
+        for (int r = 0; r < rows; ++r) {
+            const int t = c * chunk + r;
+            float cq[kScanPart], ck[kScanPart];
+            {
+                const float4* q4 = reinterpret_cast<const float4*>(buf + r * kdp + k0);
+                const float4* k4 = reinterpret_cast<const float4*>(buf + nq + r * kdp + k0);
 #pragma unroll
-            for (int i = 0; i < kScanPart; ++i) {
-                S[i] = fmaf(cb, S[i], ck[i] * w);
-                acc = fmaf(S[i], cq[i], acc);
+                for (int i = 0; i < kScanPart / 4; ++i) {
+                    const float4 a4 = q4[i], b4 = k4[i];
+                    cq[4 * i] = a4.x; cq[4 * i + 1] = a4.y; cq[4 * i + 2] = a4.z; cq[4 * i + 3] = a4.w;
+                    ck[4 * i] = b4.x; ck[4 * i + 1] = b4.y; ck[4 * i + 2] = b4.z; ck[4 * i + 3] = b4.w;
+                }
             }
-            red[t & 1][part][lane] = acc;
-            __syncthreads();
-            if (part == 0 && live) {
-                float sum = 0.f;
-                for (int p = 0; p < parts; ++p) sum += red[t & 1][p][lane];
-                op[(int64_t)t * heads * value_dim] = fmaf(d_skip, cv, sum);
-            }
-        } else {
-            // ca: the write strength, cb: the decay
+            const float cv = buf[2 * nq + r * 64 + lane];
+            const float ca = buf[2 * nq + nv + r], cb = buf[2 * nq + nv + chunk + r];
+            float acc = 0.f;
+            if (MODE == 0) {
+                // ca: the step size, cb: the decay
+                const float w = ca * cv;
 #pragma unroll
-            for (int i = 0; i < kScanPart; ++i) acc = fmaf(S[i], ck[i], acc);
-            red[0][part][lane] = acc;
-            __syncthreads();
-            float read = 0.f;
-            for (int p = 0; p < parts; ++p) read += red[0][p][lane];
-            const float u = ca * (cv - cb * read);
-            acc = 0.f;
+                for (int i = 0; i < kScanPart; ++i) {
+                    S[i] = fmaf(cb, S[i], ck[i] * w);
+                    acc = fmaf(S[i], cq[i], acc);
+                }
+                red[t & 1][part][lane] = acc;
+                __syncthreads();
+                if (part == 0) {
+                    float sum = 0.f;
+                    for (int p = 0; p < parts; ++p) sum += red[t & 1][p][lane];
+                    res[r * 64 + lane] = fmaf(d_skip, cv, sum);
+                }
+            } else {
+                // ca: the write strength, cb: the decay
 #pragma unroll
-            for (int i = 0; i < kScanPart; ++i) {
-                S[i] = fmaf(cb, S[i], ck[i] * u);
-                acc = fmaf(S[i], cq[i], acc);
+                for (int i = 0; i < kScanPart; ++i) acc = fmaf(S[i], ck[i], acc);
+                red[0][part][lane] = acc;
+                __syncthreads();
+                float read = 0.f;
+                for (int p = 0; p < parts; ++p) read += red[0][p][lane];
+                const float u = ca * (cv - cb * read);
+                acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < kScanPart; ++i) {
+                    S[i] = fmaf(cb, S[i], ck[i] * u);
+                    acc = fmaf(S[i], cq[i], acc);
+                }
+                red[1][part][lane] = acc;
+                __syncthreads();
+                if (part == 0) {
+                    float sum = 0.f;
+                    for (int p = 0; p < parts; ++p) sum += red[1][p][lane];
+                    res[r * 64 + lane] = sum;
+                }
             }
-            red[1][part][lane] = acc;
-            __syncthreads();
-            if (part == 0 && live) {
-                float sum = 0.f;
-                for (int p = 0; p < parts; ++p) sum += red[1][p][lane];
-                op[(int64_t)t * heads * value_dim] = sum;
-            }
+        }
+        // the chunk's results leave together: a store a token would make every barrier wait for memory
+        __syncthreads();
+        for (int j = tid; j < rows * 64; j += nthreads) {
+            const int r = j >> 6, cc = j & 63;
+            if (col0 + cc < value_dim) op[(int64_t)(t0 + r) * heads * value_dim + cc] = res[j];
         }
     }
     if (live) {
@@ -234,12 +282,28 @@ extern "C" int st_state_scan(float* out, const float* q, int64_t q_stride, const
              "state_scan: null operand");
     const int parts = (key_dim + kScanPart - 1) / kScanPart;
     const dim3 grid(heads, (value_dim + 63) / 64, num_items);
-    if (mode == 0)
-        state_scan_kernel<0><<<grid, 64 * parts, 0, stream>>>(out, q, q_stride, k, k_stride, v, v_stride, gate_a,
-            gate_b, skip, state, slot_stride, item_len, item_tok_off, item_slot, heads, qk_heads, key_dim, value_dim);
-    else
-        state_scan_kernel<1><<<grid, 64 * parts, 0, stream>>>(out, q, q_stride, k, k_stride, v, v_stride, gate_a,
-            gate_b, skip, state, slot_stride, item_len, item_tok_off, item_slot, heads, qk_heads, key_dim, value_dim);
+    // tokens a chunk: what 32 KB of LDS and the threads' staging registers hold
+    const int max_parts = parts <= 1 ? 1 : parts <= 2 ? 2 : parts <= 4 ? 4 : parts <= 8 ? 8 : 16;
+    int chunk = 64;
+    const int kdp = kScanPart * parts;
+    while (chunk > 1 && (4 * chunk * (2 * kdp + 66 + 64) > 40 * 1024 ||
+                         chunk * (2 * kdp + 66) > scan_regs(max_parts) * 64 * parts))
+        chunk >>= 1;
+    const size_t lds = (size_t)4 * chunk * (2 * kdp + 66 + 64);
+#define ST_SCAN(MODE, MP)                                                                                         \
+    state_scan_kernel<MODE, MP><<<grid, 64 * parts, lds, stream>>>(out, q, q_stride, k, k_stride, v, v_stride,    \
+        gate_a, gate_b, skip, state, slot_stride, item_len, item_tok_off, item_slot, heads, qk_heads, key_dim,    \
+        value_dim, chunk)
+#define ST_SCAN_MODE(MP) do { if (mode == 0) ST_SCAN(0, MP); else ST_SCAN(1, MP); } while (0)
+    switch (max_parts) {
+        case 1: ST_SCAN_MODE(1); break;
+        case 2: ST_SCAN_MODE(2); break;
+        case 4: ST_SCAN_MODE(4); break;
+        case 8: ST_SCAN_MODE(8); break;
+        default: ST_SCAN_MODE(16); break;
+    }
+#undef ST_SCAN_MODE
+#undef ST_SCAN
     ST_LAUNCH_CHECK("state_scan");
     return 0;
 }

@@ -119,5 +119,5 @@ class SinkAttention(Mixer):
 
 def K_fits(heads: int, key_dim: int, value_dim: int, mixed: bool) -> bool:
     # LDS of a workgroup: a row's queries, two blocks of scores, the mix (csrc/sink_attention.hip)
-    lds = 4 * (heads * key_dim + 2 * heads * 64 + (heads * heads if mixed else 0) + 3 * heads + 128)
+    lds = 4 * (heads * key_dim + 2 * heads * 64 + (heads * heads if mixed else 0) + 3 * heads + 1 + 256)
     return heads <= 256 and heads * value_dim <= 8192 and lds <= 64 * 1024
