@@ -10,18 +10,13 @@
 // loaded before and stored after the item's rows, so prompts, portions and single tokens take the
 // same route and a position's sums are formed in the same order however the tokens were cut.
 //
-// Launch: a workgroup a (head, block of 64 value channels, item); lane = value channel, wave = a
-// part of 16 key channels, whose column of the state stays in registers.  The waves' partial dot
-// products meet in LDS: one barrier a token for the additive form, two for the delta rule (its
-// write needs S^T k over all key channels first).  Operands are staged through LDS a chunk of
-// tokens at a time.
+// Launch: a one-wave workgroup a (head, block of 16 value channels, item), see the kernel.
 #include "api.h"
 #include "common.h"
 
 namespace st {
 
-constexpr int kScanPart = 16;        // key channels a wave
-constexpr int kScanMaxParts = 16;    // up to 256 key channels
+constexpr int kScanMaxKeys = 256;     // key channels a head: four lanes of up to 64
 
 __device__ inline float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
@@ -62,35 +57,35 @@ __global__ __launch_bounds__(256) void unit_norm_kernel(float* __restrict__ x, i
     for (int j = lane; j < dim; j += 64) p[j] *= r;
 }
 
-// Operands of `chunk` tokens at a time are staged in LDS, q [chunk, key_dim] | k [chunk, key_dim] |
-// v [chunk, 64] | a [chunk] | b [chunk], so that the walk over the tokens waits for LDS only.
-// floats a thread carries from memory to LDS for a chunk: what its register budget allows
-constexpr int scan_regs(int max_parts) { return max_parts >= 16 ? 6 : max_parts >= 8 ? 16 : 32; }
-
-template <int MODE, int MAXPARTS>
-__global__ __launch_bounds__(64 * MAXPARTS) void state_scan_kernel(
+// One wave a workgroup: lane = (quarter of the key channels, one of 16 value channels).  A lane keeps
+// its KQ key channels of its value channel's column of the state in registers; sums over the key
+// channels are sums over a lane's registers and then over the four lanes that share a value channel
+// (row swaps, no LDS, no barrier).  Operands of `chunk` tokens at a time are staged in the wave's LDS:
+// q [chunk, 4 KQ] | k [chunk, 4 KQ] (rows padded with zeros) | v [chunk, 16] | a [chunk] | b [chunk],
+// then the chunk's results [chunk, 16], which leave together.
+// VEC: rows and sizes allow 16-byte loads (the host checks alignment).
+template <int MODE, int KQ, bool VEC>
+__global__ __launch_bounds__(64) void state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
     int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ ga,
     const float* __restrict__ gb, const float* __restrict__ skip, float* __restrict__ state, int64_t slot_stride,
     const int* __restrict__ item_len, const int* __restrict__ item_tok_off, const int* __restrict__ item_slot,
     int heads, int qk_heads, int key_dim, int value_dim, int chunk) {
-    extern __shared__ __attribute__((aligned(16))) float staged[];   // a chunk's operands, then its results [chunk, 64]
-    __shared__ float red[2][kScanMaxParts][64];
+    extern __shared__ __attribute__((aligned(16))) float staged[];
+    constexpr int KW = 4 * KQ;                          // a staged row of q or k
     const int head = blockIdx.x, item = blockIdx.z;
-    const int tid = threadIdx.x, lane = tid & 63, part = tid >> 6;
-    const int nthreads = blockDim.x, parts = nthreads >> 6;
-    const int col0 = blockIdx.y * 64, col = col0 + lane;
+    const int lane = threadIdx.x, quarter = lane >> 4, vc = lane & 15;
+    const int col0 = blockIdx.y * 16, col = col0 + vc;
     const bool live = col < value_dim;
     const int slot = item_slot[item], n = item_len[item];
-    if (slot < 0 || n <= 0) return;                     // uniform over the workgroup
+    if (slot < 0 || n <= 0) return;
     const int64_t row0 = item_tok_off[item];
     const int qk_head = head / (heads / qk_heads);
-    const int k0 = part * kScanPart;
-    float S[kScanPart];
+    const int k0 = quarter * KQ;
+    float S[KQ];
     float* sp = state + (int64_t)slot * slot_stride + ((int64_t)head * key_dim + k0) * value_dim + col;
 #pragma unroll
-    for (int i = 0; i < kScanPart; ++i)
-        S[i] = (live && k0 + i < key_dim) ? sp[(int64_t)i * value_dim] : 0.f;
+    for (int i = 0; i < KQ; ++i) S[i] = (live && k0 + i < key_dim) ? sp[(int64_t)i * value_dim] : 0.f;
     const float d_skip = skip ? skip[head] : 0.f;
     const float* qp = q + row0 * q_stride + (int64_t)qk_head * key_dim;
     const float* kp = k + row0 * k_stride + (int64_t)qk_head * key_dim;
@@ -98,110 +93,141 @@ __global__ __launch_bounds__(64 * MAXPARTS) void state_scan_kernel(
     const float* ap = ga + row0 * heads + head;
     const float* bp = gb + row0 * heads + head;
     float* op = out + row0 * ((int64_t)heads * value_dim) + (int64_t)head * value_dim + col0;
-    const int kdp = kScanPart * parts;                  // a row of q or k in LDS: padded with zeros to whole parts
-    const int nq = chunk * kdp, nv = chunk * 64;
-    // A chunk's operands go to LDS through registers: all of a thread's loads are issued before any is
-    // stored, so that a chunk costs one trip to memory, not one an element.  Rows beyond the item's end
-    // are zeros.
-    const int per_buf = 2 * nq + nv + 2 * chunk;
-    float* res = staged + per_buf;
-    const int chunks = (n + chunk - 1) / chunk;
-    for (int c = 0; c < chunks; ++c) {
-        const float* buf = staged;
-        const int t0 = c * chunk;
-        constexpr int kRegs = scan_regs(MAXPARTS);
-        float pre[kRegs];
-#pragma unroll
-        for (int i = 0; i < kRegs; ++i) {
-            const int idx = tid + i * nthreads;
-            const float* src = nullptr;
-            if (idx < 2 * nq) {
-                const int j = idx < nq ? idx : idx - nq;
-                const int r = j / kdp, cc = j - r * kdp;
-                if (t0 + r < n && cc < key_dim) src = idx < nq ? qp + (int64_t)(t0 + r) * q_stride + cc : kp + (int64_t)(t0 + r) * k_stride + cc;
-            } else if (idx < 2 * nq + nv) {
-                const int j = idx - 2 * nq, r = j >> 6, cc = j & 63;
-                if (t0 + r < n && col0 + cc < value_dim) src = vp + (int64_t)(t0 + r) * v_stride + cc;
-            } else if (idx < per_buf) {
-                const int j = idx - 2 * nq - nv;
-                const int r = j < chunk ? j : j - chunk;
-                if (t0 + r < n) src = (j < chunk ? ap : bp) + (int64_t)(t0 + r) * heads;
-            }
-            pre[i] = src ? *src : 0.f;
-        }
-        __syncthreads();                     // the chunk before has been walked by every wave
-#pragma unroll
-        for (int i = 0; i < kRegs; ++i) {
-            const int idx = tid + i * nthreads;
-            if (idx < per_buf) staged[idx] = pre[i];
-        }
+    const int nq = chunk * KW, nv = chunk * 16;
+    const int total = 2 * nq + nv + 2 * chunk;
+    float* res = staged + total;
+    if (VEC) {                                          // the rows' padding beyond key_dim stays zero
+        for (int idx = lane; idx < 2 * nq; idx += 64) staged[idx] = 0.f;
         __syncthreads();
-        const int rows = min(chunk, n - c * chunk);
-        for (int r = 0; r < rows; ++r) {
-            const int t = c * chunk + r;
-            float cq[kScanPart], ck[kScanPart];
-            {
-                const float4* q4 = reinterpret_cast<const float4*>(buf + r * kdp + k0);
-                const float4* k4 = reinterpret_cast<const float4*>(buf + nq + r * kdp + k0);
+    }
+    for (int t0 = 0; t0 < n; t0 += chunk) {
+        const int rows = min(chunk, n - t0);
+        // a trip to memory costs far more than the walk over a token: as many loads a lane in flight as
+        // registers allow, then their stores; rows beyond the item's end are zeros
+        if (VEC) {
+            constexpr int NB = KQ <= 16 ? 16 : 8;
+            const int kv4 = key_dim >> 2;
+            const int nqv = chunk * kv4, nvv = chunk * 4;
+            const int totalv = 2 * nqv + nvv;
+            float gate = 0.f;
+            if (lane < 2 * chunk) {
+                const int r = lane < chunk ? lane : lane - chunk;
+                if (r < rows) gate = (lane < chunk ? ap : bp)[(int64_t)(t0 + r) * heads];
+            }
+            for (int base = 0; base < totalv; base += 64 * NB) {
+                float4 x[NB];
 #pragma unroll
-                for (int i = 0; i < kScanPart / 4; ++i) {
-                    const float4 a4 = q4[i], b4 = k4[i];
-                    cq[4 * i] = a4.x; cq[4 * i + 1] = a4.y; cq[4 * i + 2] = a4.z; cq[4 * i + 3] = a4.w;
-                    ck[4 * i] = b4.x; ck[4 * i + 1] = b4.y; ck[4 * i + 2] = b4.z; ck[4 * i + 3] = b4.w;
+                for (int u = 0; u < NB; ++u) {
+                    const int idx = base + u * 64 + lane;
+                    const float* src = nullptr;
+                    if (idx < 2 * nqv) {
+                        const int j = idx < nqv ? idx : idx - nqv;
+                        const int r = j / kv4, cc = (j - r * kv4) * 4;
+                        if (r < rows)
+                            src = idx < nqv ? qp + (int64_t)(t0 + r) * q_stride + cc : kp + (int64_t)(t0 + r) * k_stride + cc;
+                    } else if (idx < totalv) {
+                        const int j = idx - 2 * nqv, r = j >> 2, cc = (j & 3) * 4;
+                        if (r < rows && col0 + cc < value_dim) src = vp + (int64_t)(t0 + r) * v_stride + cc;
+                    }
+                    x[u] = src ? *reinterpret_cast<const float4*>(src) : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+#pragma unroll
+                for (int u = 0; u < NB; ++u) {
+                    const int idx = base + u * 64 + lane;
+                    if (idx < 2 * nqv) {
+                        const int j = idx < nqv ? idx : idx - nqv;
+                        const int r = j / kv4, cc = (j - r * kv4) * 4;
+                        *reinterpret_cast<float4*>(staged + (idx < nqv ? 0 : nq) + r * KW + cc) = x[u];
+                    } else if (idx < totalv) {
+                        *reinterpret_cast<float4*>(staged + 2 * nq + (idx - 2 * nqv) * 4) = x[u];
+                    }
                 }
             }
-            const float cv = buf[2 * nq + r * 64 + lane];
-            const float ca = buf[2 * nq + nv + r], cb = buf[2 * nq + nv + chunk + r];
-            float acc = 0.f;
+            if (lane < 2 * chunk) staged[2 * nq + nv + lane] = gate;
+        } else
+        for (int base = 0; base < total; base += 64 * 8) {
+            float x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = base + u * 64 + lane;
+                const float* src = nullptr;
+                if (idx < 2 * nq) {
+                    const int j = idx < nq ? idx : idx - nq;
+                    const int r = j / KW, cc = j % KW;
+                    if (r < rows && cc < key_dim)
+                        src = idx < nq ? qp + (int64_t)(t0 + r) * q_stride + cc : kp + (int64_t)(t0 + r) * k_stride + cc;
+                } else if (idx < 2 * nq + nv) {
+                    const int j = idx - 2 * nq, r = j >> 4, cc = j & 15;
+                    if (r < rows && col0 + cc < value_dim) src = vp + (int64_t)(t0 + r) * v_stride + cc;
+                } else if (idx < total) {
+                    const int j = idx - 2 * nq - nv;
+                    const int r = j < chunk ? j : j - chunk;
+                    if (r < rows) src = (j < chunk ? ap : bp) + (int64_t)(t0 + r) * heads;
+                }
+                x[u] = src ? *src : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = base + u * 64 + lane;
+                if (idx < total) staged[idx] = x[u];
+            }
+        }
+        __syncthreads();                                // (one wave: orders the LDS writes before the reads)
+        for (int r = 0; r < rows; ++r) {
+            float cq[KQ], ck[KQ];
+            const float4* q4 = reinterpret_cast<const float4*>(staged + r * KW + k0);
+            const float4* k4 = reinterpret_cast<const float4*>(staged + nq + r * KW + k0);
+#pragma unroll
+            for (int i = 0; i < KQ / 4; ++i) {
+                const float4 a4 = q4[i], b4 = k4[i];
+                cq[4 * i] = a4.x; cq[4 * i + 1] = a4.y; cq[4 * i + 2] = a4.z; cq[4 * i + 3] = a4.w;
+                ck[4 * i] = b4.x; ck[4 * i + 1] = b4.y; ck[4 * i + 2] = b4.z; ck[4 * i + 3] = b4.w;
+            }
+            const float cv = staged[2 * nq + r * 16 + vc];
+            const float ca = staged[2 * nq + nv + r], cb = staged[2 * nq + nv + chunk + r];
+            float o;
             if (MODE == 0) {
                 // ca: the step size, cb: the decay
                 const float w = ca * cv;
+                float acc = 0.f;
 #pragma unroll
-                for (int i = 0; i < kScanPart; ++i) {
+                for (int i = 0; i < KQ; ++i) {
                     S[i] = fmaf(cb, S[i], ck[i] * w);
                     acc = fmaf(S[i], cq[i], acc);
                 }
-                red[t & 1][part][lane] = acc;
-                __syncthreads();
-                if (part == 0) {
-                    float sum = 0.f;
-                    for (int p = 0; p < parts; ++p) sum += red[t & 1][p][lane];
-                    res[r * 64 + lane] = fmaf(d_skip, cv, sum);
-                }
+                o = fmaf(d_skip, cv, rows4_sum(acc));
             } else {
-                // ca: the write strength, cb: the decay
+                // ca: the write strength, cb: the decay.  With the state before this token, S:
+                //   u = ca (v - cb S^T k),  o = (cb S + k u^T)^T q = cb S^T q + (k . q) u:
+                // the two sums over the old state and k . q are formed in one pass
+                float rk = 0.f, rq = 0.f, kq = 0.f;
 #pragma unroll
-                for (int i = 0; i < kScanPart; ++i) acc = fmaf(S[i], ck[i], acc);
-                red[0][part][lane] = acc;
-                __syncthreads();
-                float read = 0.f;
-                for (int p = 0; p < parts; ++p) read += red[0][p][lane];
-                const float u = ca * (cv - cb * read);
-                acc = 0.f;
+                for (int i = 0; i < KQ; ++i) {
+                    rk = fmaf(S[i], ck[i], rk);
+                    rq = fmaf(S[i], cq[i], rq);
+                    kq = fmaf(ck[i], cq[i], kq);
+                }
+                rk = rows4_sum(rk);
+                rq = rows4_sum(rq);
+                kq = rows4_sum(kq);
+                const float u = ca * (cv - cb * rk);
 #pragma unroll
-                for (int i = 0; i < kScanPart; ++i) {
-                    S[i] = fmaf(cb, S[i], ck[i] * u);
-                    acc = fmaf(S[i], cq[i], acc);
-                }
-                red[1][part][lane] = acc;
-                __syncthreads();
-                if (part == 0) {
-                    float sum = 0.f;
-                    for (int p = 0; p < parts; ++p) sum += red[1][p][lane];
-                    res[r * 64 + lane] = sum;
-                }
+                for (int i = 0; i < KQ; ++i) S[i] = fmaf(cb, S[i], ck[i] * u);
+                o = fmaf(cb, rq, kq * u);
             }
+            if (quarter == 0) res[r * 16 + vc] = o;
         }
-        // the chunk's results leave together: a store a token would make every barrier wait for memory
         __syncthreads();
-        for (int j = tid; j < rows * 64; j += nthreads) {
-            const int r = j >> 6, cc = j & 63;
+        // the chunk's results leave together
+        for (int j = lane; j < rows * 16; j += 64) {
+            const int r = j >> 4, cc = j & 15;
             if (col0 + cc < value_dim) op[(int64_t)(t0 + r) * heads * value_dim + cc] = res[j];
         }
+        __syncthreads();                                // before the next chunk overwrites the buffers
     }
     if (live) {
 #pragma unroll
-        for (int i = 0; i < kScanPart; ++i)
+        for (int i = 0; i < KQ; ++i)
             if (k0 + i < key_dim) sp[(int64_t)i * value_dim] = S[i];
     }
 }
@@ -273,34 +299,35 @@ extern "C" int st_state_scan(float* out, const float* q, int64_t q_stride, const
                              int key_dim, int value_dim, int mode, hipStream_t stream) {
     ST_CHECK(num_items >= 0 && heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && key_dim > 0 && value_dim > 0,
              "state_scan: bad sizes");
-    ST_CHECK(key_dim <= kScanPart * kScanMaxParts, "state_scan: up to %d key channels a head, not %d",
-             kScanPart * kScanMaxParts, key_dim);
+    ST_CHECK(key_dim <= kScanMaxKeys, "state_scan: up to %d key channels a head, not %d", kScanMaxKeys, key_dim);
     ST_CHECK(mode == 0 || mode == 1, "state_scan: mode 0 (additive) or 1 (delta rule)");
-    ST_CHECK(num_items <= 65535 && (value_dim + 63) / 64 <= 65535, "state_scan: too many items or value channels");
+    ST_CHECK(num_items <= 65535 && (value_dim + 15) / 16 <= 65535, "state_scan: too many items or value channels");
     if (num_items == 0) return 0;
     ST_CHECK(out && q && k && v && gate_a && gate_b && state && item_len && item_tok_off && item_slot,
              "state_scan: null operand");
-    const int parts = (key_dim + kScanPart - 1) / kScanPart;
-    const dim3 grid(heads, (value_dim + 63) / 64, num_items);
-    // tokens a chunk: what 32 KB of LDS and the threads' staging registers hold
-    const int max_parts = parts <= 1 ? 1 : parts <= 2 ? 2 : parts <= 4 ? 4 : parts <= 8 ? 8 : 16;
-    int chunk = 64;
-    const int kdp = kScanPart * parts;
-    while (chunk > 1 && (4 * chunk * (2 * kdp + 66 + 64) > 40 * 1024 ||
-                         chunk * (2 * kdp + 66) > scan_regs(max_parts) * 64 * parts))
-        chunk >>= 1;
-    const size_t lds = (size_t)4 * chunk * (2 * kdp + 66 + 64);
-#define ST_SCAN(MODE, MP)                                                                                         \
-    state_scan_kernel<MODE, MP><<<grid, 64 * parts, lds, stream>>>(out, q, q_stride, k, k_stride, v, v_stride,    \
-        gate_a, gate_b, skip, state, slot_stride, item_len, item_tok_off, item_slot, heads, qk_heads, key_dim,    \
+    // key channels a lane: a quarter of the head's, rounded up to a power of two from 4 on
+    int kq = 4;
+    while (4 * kq < key_dim) kq <<= 1;
+    const dim3 grid(heads, (value_dim + 15) / 16, num_items);
+    // tokens a chunk: what 24 KB of LDS hold
+    int chunk = 32;
+    while (chunk > 1 && 4 * chunk * (8 * kq + 18 + 16) > 24 * 1024) chunk >>= 1;
+    const size_t lds = (size_t)4 * chunk * (8 * kq + 18 + 16);
+    // 16-byte loads where every row of q, k and v starts on a 16-byte border and the sizes are whole fours
+    const bool vec = key_dim % 4 == 0 && value_dim % 4 == 0 && q_stride % 4 == 0 && k_stride % 4 == 0 &&
+                     v_stride % 4 == 0 && (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0;
+#define ST_SCAN(MODE, KQ, VEC)                                                                                      \
+    state_scan_kernel<MODE, KQ, VEC><<<grid, 64, lds, stream>>>(out, q, q_stride, k, k_stride, v, v_stride, gate_a, \
+        gate_b, skip, state, slot_stride, item_len, item_tok_off, item_slot, heads, qk_heads, key_dim,              \
         value_dim, chunk)
-#define ST_SCAN_MODE(MP) do { if (mode == 0) ST_SCAN(0, MP); else ST_SCAN(1, MP); } while (0)
-    switch (max_parts) {
-        case 1: ST_SCAN_MODE(1); break;
-        case 2: ST_SCAN_MODE(2); break;
+#define ST_SCAN_MODE(KQ) do { if (mode == 0) { if (vec) ST_SCAN(0, KQ, true); else ST_SCAN(0, KQ, false); }        \
+                              else { if (vec) ST_SCAN(1, KQ, true); else ST_SCAN(1, KQ, false); } } while (0)
+    switch (kq) {
         case 4: ST_SCAN_MODE(4); break;
         case 8: ST_SCAN_MODE(8); break;
-        default: ST_SCAN_MODE(16); break;
+        case 16: ST_SCAN_MODE(16); break;
+        case 32: ST_SCAN_MODE(32); break;
+        default: ST_SCAN_MODE(64); break;
     }
 #undef ST_SCAN_MODE
 #undef ST_SCAN
