@@ -100,8 +100,13 @@ class SinkAttention(Mixer):
         blocks = max(1, -(-span // 64))
         return max(1, min(256 // max(rows, 1), blocks, 16))
 
-    def forward(self, x_t: torch.Tensor, residual32: torch.Tensor, ctx, cache, write: bool = True) -> torch.Tensor:
-        qkv = K.gemm(x_t, self.w_qkv, bias=self.b_qkv)
+    accepts_norm = True     # forward(..., norm=part) normalises residual32 itself
+
+    def forward(self, x_t: Optional[torch.Tensor], residual32: torch.Tensor, ctx, cache, write: bool = True,
+                norm=None) -> torch.Tensor:
+        """residual32 + mix(x_t).  With ``norm`` (a norm part that offers ``as_input``), the mixer's input is
+        norm(residual32), computed inside the QKV product."""
+        qkv = K.gemm(norm.as_input(residual32) if norm is not None else x_t, self.w_qkv, bias=self.b_qkv)
         q = qkv[:, :self.q_size]
         k = qkv[:, self.q_size:self.q_size + self.k_size]
         v = qkv[:, self.q_size + self.k_size:]
