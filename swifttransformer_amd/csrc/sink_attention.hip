@@ -268,7 +268,10 @@ __global__ __launch_bounds__(256) void sink_attention_merge_kernel(
     for (int e = threadIdx.x; e < width; e += 256) {
         const float* w = wgt + (e / value_dim) * splits;
         float num = 0.f;
-        for (int s = 0; s < splits; ++s) num = fmaf(w[s], po[(int64_t)s * width + e], num);
+        for (int s = 0; s < splits; ++s) {
+            const float x = po[(int64_t)s * width + e];      // (a split without keys may hold anything)
+            num = fmaf(w[s], w[s] > 0.f ? x : 0.f, num);
+        }
         Elem<T>::store(out + (int64_t)t * width + e, num);
     }
 }
