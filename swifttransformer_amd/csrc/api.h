@@ -148,7 +148,8 @@ int st_unit_norm(float* x, int64_t stride, int num_tokens, int heads, int dim, f
 int st_state_scan(float* out, const float* q, int64_t q_stride, const float* k, int64_t k_stride, const float* v,
                   int64_t v_stride, const float* gate_a, const float* gate_b, const float* skip, float* state,
                   int64_t slot_stride, const int* item_len, const int* item_tok_off, const int* item_slot,
-                  int num_items, int heads, int qk_heads, int key_dim, int value_dim, int mode, hipStream_t stream);
+                  int num_items, int max_item_rows, int heads, int qk_heads, int key_dim, int value_dim, int mode,
+                  hipStream_t stream);
 // out = val * rsqrt(mean(val^2) + eps) * gain (* silu(gate) unless gate_first) over each of `groups`
 // parts of a row, val = o (* silu(gate) if gate_first); gain [width], or [groups * width] if gain_per_group.
 int st_gated_group_norm(void* out, const float* o, const void* gate, int64_t gate_stride, const float* gain,

@@ -10,7 +10,7 @@
 // loaded before and stored after the item's rows, so prompts, portions and single tokens take the
 // same route and a position's sums are formed in the same order however the tokens were cut.
 //
-// Launch: a one-wave workgroup a (head, block of 16 value channels, item), see the kernel.
+// Launch: a two-wave workgroup a (head, block of 16 value channels, item), see the kernel.
 #include "api.h"
 #include "common.h"
 
@@ -57,15 +57,17 @@ __global__ __launch_bounds__(256) void unit_norm_kernel(float* __restrict__ x, i
     for (int j = lane; j < dim; j += 64) p[j] *= r;
 }
 
-// One wave a workgroup: lane = (quarter of the key channels, one of 16 value channels).  A lane keeps
-// its KQ key channels of its value channel's column of the state in registers; sums over the key
-// channels are sums over a lane's registers and then over the four lanes that share a value channel
-// (row swaps, no LDS, no barrier).  Operands of `chunk` tokens at a time are staged in the wave's LDS:
-// q [chunk, 4 KQ] | k [chunk, 4 KQ] (rows padded with zeros) | v [chunk, 16] | a [chunk] | b [chunk],
-// then the chunk's results [chunk, 16], which leave together.
+// Two waves a workgroup.  The walker: lane = (quarter of the key channels, one of 16 value channels); a
+// lane keeps its KQ key channels of its value channel's column of the state in registers; sums over the
+// key channels are sums over a lane's registers and then over the four lanes that share a value channel
+// (row swaps, no LDS traffic between lanes).  The loader stages the operands of the next `chunk` tokens
+// in LDS while the walker walks the current chunk, and stores the results of the chunk before: a trip to
+// memory costs as much as the walk over a dozen tokens, and this way the walker waits for none.  The two
+// meet at one barrier a chunk.  A staging buffer: q [chunk, 4 KQ] | k [chunk, 4 KQ] (rows padded with
+// zeros) | v [chunk, 16] | a [chunk] | b [chunk]; two of them, then two result buffers [chunk, 16].
 // VEC: rows and sizes allow 16-byte loads (the host checks alignment).
 template <int MODE, int KQ, bool VEC>
-__global__ __launch_bounds__(64) void state_scan_kernel(
+__global__ __launch_bounds__(128) void state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
     int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ ga,
     const float* __restrict__ gb, const float* __restrict__ skip, float* __restrict__ state, int64_t slot_stride,
@@ -74,19 +76,16 @@ __global__ __launch_bounds__(64) void state_scan_kernel(
     extern __shared__ __attribute__((aligned(16))) float staged[];
     constexpr int KW = 4 * KQ;                          // a staged row of q or k
     const int head = blockIdx.x, item = blockIdx.z;
-    const int lane = threadIdx.x, quarter = lane >> 4, vc = lane & 15;
+    const int lane = threadIdx.x & 63;
+    const bool loader = threadIdx.x >= 64;
+    const int quarter = lane >> 4, vc = lane & 15;
     const int col0 = blockIdx.y * 16, col = col0 + vc;
     const bool live = col < value_dim;
     const int slot = item_slot[item], n = item_len[item];
-    if (slot < 0 || n <= 0) return;
+    if (slot < 0 || n <= 0) return;                     // uniform over the workgroup
     const int64_t row0 = item_tok_off[item];
     const int qk_head = head / (heads / qk_heads);
     const int k0 = quarter * KQ;
-    float S[KQ];
-    float* sp = state + (int64_t)slot * slot_stride + ((int64_t)head * key_dim + k0) * value_dim + col;
-#pragma unroll
-    for (int i = 0; i < KQ; ++i) S[i] = (live && k0 + i < key_dim) ? sp[(int64_t)i * value_dim] : 0.f;
-    const float d_skip = skip ? skip[head] : 0.f;
     const float* qp = q + row0 * q_stride + (int64_t)qk_head * key_dim;
     const float* kp = k + row0 * k_stride + (int64_t)qk_head * key_dim;
     const float* vp = v + row0 * v_stride + (int64_t)head * value_dim + col0;
@@ -94,21 +93,18 @@ __global__ __launch_bounds__(64) void state_scan_kernel(
     const float* bp = gb + row0 * heads + head;
     float* op = out + row0 * ((int64_t)heads * value_dim) + (int64_t)head * value_dim + col0;
     const int nq = chunk * KW, nv = chunk * 16;
-    const int total = 2 * nq + nv + 2 * chunk;
-    float* res = staged + total;
-    if (VEC) {                                          // the rows' padding beyond key_dim stays zero
-        for (int idx = lane; idx < 2 * nq; idx += 64) staged[idx] = 0.f;
-        __syncthreads();
-    }
-    for (int t0 = 0; t0 < n; t0 += chunk) {
-        const int rows = min(chunk, n - t0);
-        // a trip to memory costs far more than the walk over a token: as many loads a lane in flight as
-        // registers allow, then their stores; rows beyond the item's end are zeros
+    const int total = 2 * nq + nv + 2 * chunk;          // floats of a staging buffer
+    float* res_base = staged + 2 * total;
+    const int chunks = (n + chunk - 1) / chunk;
+
+    // the loader's two jobs (its 64 lanes)
+    auto stage = [&](int c) {
+        float* buf = staged + (c & 1) * total;
+        const int t0 = c * chunk, rows = min(chunk, n - t0);
         if (VEC) {
-            constexpr int NB = KQ <= 16 ? 16 : 8;
+            constexpr int NB = KQ <= 16 ? 16 : 8;       // 16-byte loads a lane in flight
             const int kv4 = key_dim >> 2;
-            const int nqv = chunk * kv4, nvv = chunk * 4;
-            const int totalv = 2 * nqv + nvv;
+            const int nqv = chunk * kv4, totalv = 2 * nqv + chunk * 4;
             float gate = 0.f;
             if (lane < 2 * chunk) {
                 const int r = lane < chunk ? lane : lane - chunk;
@@ -137,95 +133,124 @@ __global__ __launch_bounds__(64) void state_scan_kernel(
                     if (idx < 2 * nqv) {
                         const int j = idx < nqv ? idx : idx - nqv;
                         const int r = j / kv4, cc = (j - r * kv4) * 4;
-                        *reinterpret_cast<float4*>(staged + (idx < nqv ? 0 : nq) + r * KW + cc) = x[u];
+                        *reinterpret_cast<float4*>(buf + (idx < nqv ? 0 : nq) + r * KW + cc) = x[u];
                     } else if (idx < totalv) {
-                        *reinterpret_cast<float4*>(staged + 2 * nq + (idx - 2 * nqv) * 4) = x[u];
+                        *reinterpret_cast<float4*>(buf + 2 * nq + (idx - 2 * nqv) * 4) = x[u];
                     }
                 }
             }
-            if (lane < 2 * chunk) staged[2 * nq + nv + lane] = gate;
-        } else
-        for (int base = 0; base < total; base += 64 * 8) {
-            float x[8];
+            if (lane < 2 * chunk) buf[2 * nq + nv + lane] = gate;
+        } else {
+            for (int base = 0; base < total; base += 64 * 8) {
+                float x[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int idx = base + u * 64 + lane;
-                const float* src = nullptr;
-                if (idx < 2 * nq) {
-                    const int j = idx < nq ? idx : idx - nq;
-                    const int r = j / KW, cc = j % KW;
-                    if (r < rows && cc < key_dim)
-                        src = idx < nq ? qp + (int64_t)(t0 + r) * q_stride + cc : kp + (int64_t)(t0 + r) * k_stride + cc;
-                } else if (idx < 2 * nq + nv) {
-                    const int j = idx - 2 * nq, r = j >> 4, cc = j & 15;
-                    if (r < rows && col0 + cc < value_dim) src = vp + (int64_t)(t0 + r) * v_stride + cc;
-                } else if (idx < total) {
-                    const int j = idx - 2 * nq - nv;
-                    const int r = j < chunk ? j : j - chunk;
-                    if (r < rows) src = (j < chunk ? ap : bp) + (int64_t)(t0 + r) * heads;
+                for (int u = 0; u < 8; ++u) {
+                    const int idx = base + u * 64 + lane;
+                    const float* src = nullptr;
+                    if (idx < 2 * nq) {
+                        const int j = idx < nq ? idx : idx - nq;
+                        const int r = j / KW, cc = j % KW;
+                        if (r < rows && cc < key_dim)
+                            src = idx < nq ? qp + (int64_t)(t0 + r) * q_stride + cc : kp + (int64_t)(t0 + r) * k_stride + cc;
+                    } else if (idx < 2 * nq + nv) {
+                        const int j = idx - 2 * nq, r = j >> 4, cc = j & 15;
+                        if (r < rows && col0 + cc < value_dim) src = vp + (int64_t)(t0 + r) * v_stride + cc;
+                    } else if (idx < total) {
+                        const int j = idx - 2 * nq - nv;
+                        const int r = j < chunk ? j : j - chunk;
+                        if (r < rows) src = (j < chunk ? ap : bp) + (int64_t)(t0 + r) * heads;
+                    }
+                    x[u] = src ? *src : 0.f;
                 }
-                x[u] = src ? *src : 0.f;
-            }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int idx = base + u * 64 + lane;
-                if (idx < total) staged[idx] = x[u];
+                for (int u = 0; u < 8; ++u) {
+                    const int idx = base + u * 64 + lane;
+                    if (idx < total) buf[idx] = x[u];
+                }
             }
         }
-        __syncthreads();                                // (one wave: orders the LDS writes before the reads)
-        for (int r = 0; r < rows; ++r) {
-            float cq[KQ], ck[KQ];
-            const float4* q4 = reinterpret_cast<const float4*>(staged + r * KW + k0);
-            const float4* k4 = reinterpret_cast<const float4*>(staged + nq + r * KW + k0);
-#pragma unroll
-            for (int i = 0; i < KQ / 4; ++i) {
-                const float4 a4 = q4[i], b4 = k4[i];
-                cq[4 * i] = a4.x; cq[4 * i + 1] = a4.y; cq[4 * i + 2] = a4.z; cq[4 * i + 3] = a4.w;
-                ck[4 * i] = b4.x; ck[4 * i + 1] = b4.y; ck[4 * i + 2] = b4.z; ck[4 * i + 3] = b4.w;
-            }
-            const float cv = staged[2 * nq + r * 16 + vc];
-            const float ca = staged[2 * nq + nv + r], cb = staged[2 * nq + nv + chunk + r];
-            float o;
-            if (MODE == 0) {
-                // ca: the step size, cb: the decay
-                const float w = ca * cv;
-                float acc = 0.f;
-#pragma unroll
-                for (int i = 0; i < KQ; ++i) {
-                    S[i] = fmaf(cb, S[i], ck[i] * w);
-                    acc = fmaf(S[i], cq[i], acc);
-                }
-                o = fmaf(d_skip, cv, rows4_sum(acc));
-            } else {
-                // ca: the write strength, cb: the decay.  With the state before this token, S:
-                //   u = ca (v - cb S^T k),  o = (cb S + k u^T)^T q = cb S^T q + (k . q) u:
-                // the two sums over the old state and k . q are formed in one pass
-                float rk = 0.f, rq = 0.f, kq = 0.f;
-#pragma unroll
-                for (int i = 0; i < KQ; ++i) {
-                    rk = fmaf(S[i], ck[i], rk);
-                    rq = fmaf(S[i], cq[i], rq);
-                    kq = fmaf(ck[i], cq[i], kq);
-                }
-                rk = rows4_sum(rk);
-                rq = rows4_sum(rq);
-                kq = rows4_sum(kq);
-                const float u = ca * (cv - cb * rk);
-#pragma unroll
-                for (int i = 0; i < KQ; ++i) S[i] = fmaf(cb, S[i], ck[i] * u);
-                o = fmaf(cb, rq, kq * u);
-            }
-            if (quarter == 0) res[r * 16 + vc] = o;
-        }
-        __syncthreads();
-        // the chunk's results leave together
+    };
+    auto store_results = [&](int c) {
+        const float* res = res_base + (c & 1) * nv;
+        const int t0 = c * chunk, rows = min(chunk, n - t0);
         for (int j = lane; j < rows * 16; j += 64) {
             const int r = j >> 4, cc = j & 15;
             if (col0 + cc < value_dim) op[(int64_t)(t0 + r) * heads * value_dim + cc] = res[j];
         }
-        __syncthreads();                                // before the next chunk overwrites the buffers
+    };
+
+    // the walker's state
+    float S[KQ];
+    float* sp = state + (int64_t)slot * slot_stride + ((int64_t)head * key_dim + k0) * value_dim + col;
+    float d_skip = 0.f;
+    if (!loader) {
+#pragma unroll
+        for (int i = 0; i < KQ; ++i) S[i] = (live && k0 + i < key_dim) ? sp[(int64_t)i * value_dim] : 0.f;
+        d_skip = skip ? skip[head] : 0.f;
+    } else {
+        if (VEC && key_dim < KW)                         // the rows' padding beyond key_dim stays zero in both buffers
+            for (int idx = lane; idx < 2 * total; idx += 64) staged[idx] = 0.f;
+        stage(0);
     }
-    if (live) {
+    __syncthreads();
+    for (int c = 0; c < chunks; ++c) {
+        if (loader) {
+            if (c + 1 < chunks) stage(c + 1);           // the buffer the walker left a chunk ago
+            if (c > 0) store_results(c - 1);
+        } else {
+            const float* buf = staged + (c & 1) * total;
+            float* res = res_base + (c & 1) * nv;
+            const int rows = min(chunk, n - c * chunk);
+            for (int r = 0; r < rows; ++r) {
+                float cq[KQ], ck[KQ];
+                const float4* q4 = reinterpret_cast<const float4*>(buf + r * KW + k0);
+                const float4* k4 = reinterpret_cast<const float4*>(buf + nq + r * KW + k0);
+#pragma unroll
+                for (int i = 0; i < KQ / 4; ++i) {
+                    const float4 a4 = q4[i], b4 = k4[i];
+                    cq[4 * i] = a4.x; cq[4 * i + 1] = a4.y; cq[4 * i + 2] = a4.z; cq[4 * i + 3] = a4.w;
+                    ck[4 * i] = b4.x; ck[4 * i + 1] = b4.y; ck[4 * i + 2] = b4.z; ck[4 * i + 3] = b4.w;
+                }
+                const float cv = buf[2 * nq + r * 16 + vc];
+                const float ca = buf[2 * nq + nv + r], cb = buf[2 * nq + nv + chunk + r];
+                float o;
+                if (MODE == 0) {
+                    // ca: the step size, cb: the decay
+                    const float w = ca * cv;
+                    float acc = 0.f;
+#pragma unroll
+                    for (int i = 0; i < KQ; ++i) {
+                        S[i] = fmaf(cb, S[i], ck[i] * w);
+                        acc = fmaf(S[i], cq[i], acc);
+                    }
+                    o = fmaf(d_skip, cv, rows4_sum(acc));
+                } else {
+                    // ca: the write strength, cb: the decay.  With the state before this token, S:
+                    //   u = ca (v - cb S^T k),  o = (cb S + k u^T)^T q = cb S^T q + (k . q) u:
+                    // the two sums over the old state and k . q are formed in one pass
+                    float rk = 0.f, rq = 0.f, kq = 0.f;
+#pragma unroll
+                    for (int i = 0; i < KQ; ++i) {
+                        rk = fmaf(S[i], ck[i], rk);
+                        rq = fmaf(S[i], cq[i], rq);
+                        kq = fmaf(ck[i], cq[i], kq);
+                    }
+                    rk = rows4_sum(rk);
+                    rq = rows4_sum(rq);
+                    kq = rows4_sum(kq);
+                    const float u = ca * (cv - cb * rk);
+#pragma unroll
+                    for (int i = 0; i < KQ; ++i) S[i] = fmaf(cb, S[i], ck[i] * u);
+                    o = fmaf(cb, rq, kq * u);
+                }
+                if (quarter == 0) res[r * 16 + vc] = o;
+            }
+        }
+        __syncthreads();
+    }
+    if (loader) {
+        store_results(chunks - 1);
+    } else if (live) {
 #pragma unroll
         for (int i = 0; i < KQ; ++i)
             if (k0 + i < key_dim) sp[(int64_t)i * value_dim] = S[i];
@@ -295,8 +320,8 @@ extern "C" int st_unit_norm(float* x, int64_t stride, int num_tokens, int heads,
 extern "C" int st_state_scan(float* out, const float* q, int64_t q_stride, const float* k, int64_t k_stride,
                              const float* v, int64_t v_stride, const float* gate_a, const float* gate_b,
                              const float* skip, float* state, int64_t slot_stride, const int* item_len,
-                             const int* item_tok_off, const int* item_slot, int num_items, int heads, int qk_heads,
-                             int key_dim, int value_dim, int mode, hipStream_t stream) {
+                             const int* item_tok_off, const int* item_slot, int num_items, int max_item_rows, int heads,
+                             int qk_heads, int key_dim, int value_dim, int mode, hipStream_t stream) {
     ST_CHECK(num_items >= 0 && heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && key_dim > 0 && value_dim > 0,
              "state_scan: bad sizes");
     ST_CHECK(key_dim <= kScanMaxKeys, "state_scan: up to %d key channels a head, not %d", kScanMaxKeys, key_dim);
@@ -309,15 +334,16 @@ extern "C" int st_state_scan(float* out, const float* q, int64_t q_stride, const
     int kq = 4;
     while (4 * kq < key_dim) kq <<= 1;
     const dim3 grid(heads, (value_dim + 15) / 16, num_items);
-    // tokens a chunk: what 24 KB of LDS hold
+    // tokens a chunk (at most 32: a lane a gate value): two staging buffers and two result buffers in 48 KB of LDS
+    // and no more than an item's rows can be (the caller's bound): steps of single tokens stage little
     int chunk = 32;
-    while (chunk > 1 && 4 * chunk * (8 * kq + 18 + 16) > 24 * 1024) chunk >>= 1;
-    const size_t lds = (size_t)4 * chunk * (8 * kq + 18 + 16);
+    while (chunk > 2 && (2 * 4 * chunk * (8 * kq + 18 + 16) > 48 * 1024 || chunk >= 2 * max_item_rows)) chunk >>= 1;
+    const size_t lds = (size_t)2 * 4 * chunk * (8 * kq + 18 + 16);
     // 16-byte loads where every row of q, k and v starts on a 16-byte border and the sizes are whole fours
     const bool vec = key_dim % 4 == 0 && value_dim % 4 == 0 && q_stride % 4 == 0 && k_stride % 4 == 0 &&
                      v_stride % 4 == 0 && (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0;
 #define ST_SCAN(MODE, KQ, VEC)                                                                                      \
-    state_scan_kernel<MODE, KQ, VEC><<<grid, 64, lds, stream>>>(out, q, q_stride, k, k_stride, v, v_stride, gate_a, \
+    state_scan_kernel<MODE, KQ, VEC><<<grid, 128, lds, stream>>>(out, q, q_stride, k, k_stride, v, v_stride, gate_a, \
         gate_b, skip, state, slot_stride, item_len, item_tok_off, item_slot, heads, qk_heads, key_dim,              \
         value_dim, chunk)
 #define ST_SCAN_MODE(KQ) do { if (mode == 0) { if (vec) ST_SCAN(0, KQ, true); else ST_SCAN(0, KQ, false); }        \

@@ -82,7 +82,7 @@ def _lib():
         lib.st_recurrence_gates.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int, _c_int, _c_int, _c_p]
         lib.st_unit_norm.argtypes = [_c_p, _c_i64, _c_int, _c_int, _c_int, _c_f, _c_f, _c_p]
         lib.st_state_scan.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_i64,
-                                      _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
+                                      _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_gated_group_norm.argtypes = [_c_p, _c_p, _c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                             _c_f, _c_int, _c_p]
         lib.st_decay_gate.argtypes = [_c_p, _c_p, _c_i64, _c_f, _c_p]
@@ -943,7 +943,7 @@ def unit_norm(x: torch.Tensor, heads: int, eps: float, scale: float = 1.0) -> to
     return x
 
 
-def _d_state_scan(q, k, v, gate_a, gate_b, state, ctx_arrays, heads, mode, skip=None):
+def _d_state_scan(q, k, v, gate_a, gate_b, state, ctx_arrays, heads, mode, skip=None, max_item_rows=0):
     T = q.shape[0]
     vd = v.shape[1] // heads
     kd = state.shape[2]
@@ -955,15 +955,17 @@ def _d_state_scan(q, k, v, gate_a, gate_b, state, ctx_arrays, heads, mode, skip=
 
 @_timed("state_scan", _d_state_scan)
 def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate_a: torch.Tensor, gate_b: torch.Tensor,
-               state: torch.Tensor, ctx_arrays, heads: int, mode: str, skip: Optional[torch.Tensor] = None) -> torch.Tensor:
+               state: torch.Tensor, ctx_arrays, heads: int, mode: str, skip: Optional[torch.Tensor] = None,
+               max_item_rows: int = 0) -> torch.Tensor:
     """Per item and head, from the slot's state S [key_dim, value_dim] and over the item's rows in order
     (a = gate_a[t, head], b = gate_b[t, head]):
     ``"additive"``: S <- b S + (a k_t) v_t^T, o_t = S^T q_t + skip[head] v_t;
     ``"delta"``: S <- b S, u = a (v_t - S^T k_t), S <- S + k_t u^T, o_t = S^T q_t.
     The state is stored back.  q, k: float [T, qk_heads * key_dim], v: float [T, heads * value_dim] (dense
     rows, any stride; head h reads q/k head h // (heads / qk_heads)); state: float
-    [slots, heads, key_dim, value_dim] (slots may be parts of a larger per-slot state).  Returns float
-    [T, heads * value_dim]."""
+    [slots, heads, key_dim, value_dim] (slots may be parts of a larger per-slot state).  ``max_item_rows``: a
+    bound on the rows of any item where the caller knows one (1 in steps of single tokens; 0: the launch's
+    rows); it sizes the kernel's staging, nothing else.  Returns float [T, heads * value_dim]."""
     _token_item, item_len, item_tok_off, item_slot = ctx_arrays
     T = q.shape[0]
     _, sh, kd, vd = state.shape
@@ -987,7 +989,7 @@ def state_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate_a: torch.
     out = empty((T, heads * vd), torch.float32, q.device)
     _check(_lib().st_state_scan(_ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0),
                                 _ptr(gate_a), _ptr(gate_b), _ptr(skip), _ptr(state), slot_stride, _ptr(item_len),
-                                _ptr(item_tok_off), _ptr(item_slot), B, heads, qk_heads, kd, vd,
+                                _ptr(item_tok_off), _ptr(item_slot), B, int(max_item_rows) or T, heads, qk_heads, kd, vd,
                                 {"additive": 0, "delta": 1}[mode], _stream()))
     return out
 

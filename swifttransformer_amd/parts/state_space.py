@@ -112,7 +112,7 @@ class Mamba2Mixer(_RecurrentMixer):
         xbc = K.token_conv(proj[:, inner:], self.w_conv, conv_state, items, torch.float32, add_input=False,
                            bias=self.b_conv, activation="silu")
         y = K.state_scan(xbc[:, inner + bc:], xbc[:, inner:inner + bc], xbc[:, :inner], steps, decay, state, items,
-                         self.num_heads, "additive", skip=self.skip)
+                         self.num_heads, "additive", skip=self.skip, max_item_rows=1 if ctx.all_single else 0)
         g = K.gated_group_norm(y, proj[:, :inner], self.gain, self.norm_groups, self.eps, self.dtype, gate_first=True)
         return K.gemm(g, self.w_out, residual=residual32, out_f32=True)
 
@@ -184,6 +184,6 @@ class GatedDeltaRule(_RecurrentMixer):
         K.unit_norm(qkv[:, :qk], self.num_qk_heads, self.unit_eps, float(self.key_dim) ** -0.5)
         K.unit_norm(qkv[:, qk:2 * qk], self.num_qk_heads, self.unit_eps)
         o = K.state_scan(qkv[:, :qk], qkv[:, qk:2 * qk], qkv[:, 2 * qk:], strength, decay, state, items,
-                         self.num_heads, "delta")
+                         self.num_heads, "delta", max_item_rows=1 if ctx.all_single else 0)
         y = K.gated_group_norm(o, proj[:, c:], self.gain, self.num_heads, self.eps, self.dtype)
         return K.gemm(y, self.w_out, residual=residual32, out_f32=True)
