@@ -55,9 +55,18 @@ __device__ inline void dot_rows(const float* __restrict__ qs, int q_stride, cons
                 float kv[V];
                 Elem<T>::unpack(raw[u], kv);
 #pragma unroll
-                for (int n = 0; n < NQ; ++n)
+                for (int n = 0; n < NQ; ++n) {
+                    // (the queries lie on 16-byte borders in LDS: dim is a multiple of four here)
+                    const float4* q4 = reinterpret_cast<const float4*>(qs + n * q_stride + d + u * V);
 #pragma unroll
-                    for (int i = 0; i < V; ++i) acc[n] = fmaf(qs[n * q_stride + d + u * V + i], kv[i], acc[n]);
+                    for (int i = 0; i < V / 4; ++i) {
+                        const float4 qv = q4[i];
+                        acc[n] = fmaf(qv.x, kv[4 * i], acc[n]);
+                        acc[n] = fmaf(qv.y, kv[4 * i + 1], acc[n]);
+                        acc[n] = fmaf(qv.z, kv[4 * i + 2], acc[n]);
+                        acc[n] = fmaf(qv.w, kv[4 * i + 3], acc[n]);
+                    }
+                }
             }
         }
         for (; d < dim; d += V) {
@@ -81,7 +90,7 @@ __device__ inline void dot_rows(const float* __restrict__ qs, int q_stride, cons
 // where the value size is a multiple of that)
 template <typename T, int NG, int W>
 __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
-    extern __shared__ float lds[];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
     const int H = a.heads, G = a.kv_heads, dk = a.key_dim, dv = a.value_dim, per = a.heads / a.kv_heads;
     float* qs = lds;                               // [H * dk]
     float* sraw = qs + H * dk;                     // [H * 64]
@@ -162,6 +171,31 @@ __global__ __launch_bounds__(256) void sink_attention_kernel(SinkAttnArgs a) {
             }
         }
         __syncthreads();
+        if (a.mix && H % 4 == 0) {
+            // a thread's outputs share its key (the lane) and differ in the head (wave + 4 i): the key's
+            // products are read once four heads at a time, the mix's rows in 16-byte pieces
+            const int jj = lane, nout = H >> 2;
+            for (int i0 = 0; i0 < nout; i0 += 8) {
+                float acc[8];
+#pragma unroll
+                for (int ii = 0; ii < 8; ++ii) acc[ii] = 0.f;
+                for (int g0 = 0; g0 < H; g0 += 4) {
+                    const float s0 = sraw[g0 * kKeyBlock + jj], s1 = sraw[(g0 + 1) * kKeyBlock + jj];
+                    const float s2 = sraw[(g0 + 2) * kKeyBlock + jj], s3 = sraw[(g0 + 3) * kKeyBlock + jj];
+#pragma unroll
+                    for (int ii = 0; ii < 8; ++ii) {
+                        if (i0 + ii < nout) {
+                            const int h = wave + 4 * (i0 + ii);
+                            const float4 m = *reinterpret_cast<const float4*>(mix_s + h * H + g0);
+                            acc[ii] = fmaf(m.w, s3, fmaf(m.z, s2, fmaf(m.y, s1, fmaf(m.x, s0, acc[ii]))));
+                        }
+                    }
+                }
+#pragma unroll
+                for (int ii = 0; ii < 8; ++ii)
+                    if (i0 + ii < nout) smix[(wave + 4 * (i0 + ii)) * kKeyBlock + jj] = jj < nk ? acc[ii] : -INFINITY;
+            }
+        } else
         for (int p = tid; p < H * kKeyBlock; p += 256) {
             const int h = p >> 6, jj = p & 63;
             float s = -INFINITY;
